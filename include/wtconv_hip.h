@@ -1,0 +1,130 @@
+/*
+ * wtconv_hip.h -- C ABI of libwtconv_hip.so: the WTConv layer (wavelet convolution,
+ * Haar/db1) forward and backward as hand-written gfx950 HIP kernels.
+ *
+ * Conventions (all entry points):
+ *   - every pointer except the parameter/gradient tables is DEVICE memory owned by the
+ *     caller; the library never allocates, frees or synchronises, and launches on the
+ *     HIP stream handed in (`stream`, a hipStream_t passed as void*; NULL = default);
+ *   - activations are contiguous NCHW (2-D) / NCL (1-D) in `dtype`; parameters are
+ *     contiguous in `param_dtype`; parameter gradients are always written as float;
+ *   - return value 0 on success, a negative WTCONV_E_* code otherwise, with a message
+ *     retrievable from wtconv_last_error() on the calling thread;
+ *   - `workspace` must hold at least wtconv*_workspace_bytes(...) bytes, 256-byte aligned.
+ *
+ * This boundary takes the place of the reference's pybind11 extension module
+ * (fast_wtconv/cuda_haar/haar.cpp:5-39), whose six functions are likewise
+ * caller-allocates / out-parameter style and launch on the current stream.
+ */
+#ifndef WTCONV_HIP_H
+#define WTCONV_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WTCONV_MAX_LEVELS 5
+#define WTCONV_ABI_VERSION 1
+
+enum { WTCONV_F32 = 0, WTCONV_BF16 = 1 };
+
+enum {
+  WTCONV_OK = 0,
+  WTCONV_E_ARG = -1,        /* bad shape / dtype / null pointer / alignment          */
+  WTCONV_E_UNSUPPORTED = -2,/* kernel size or plane too large for the built kernels  */
+  WTCONV_E_WORKSPACE = -3,  /* workspace too small                                   */
+  WTCONV_E_LAUNCH = -4      /* HIP reported a launch error                           */
+};
+
+enum { WTCONV_PASS_FORWARD = 0, WTCONV_PASS_BACKWARD_INPUT = 1, WTCONV_PASS_BACKWARD_PARAMS = 2 };
+
+/* Device pointers to the layer's parameters, in the reference module's own tensor
+ * layouts (wtconv/wtconv2d.py:23-31, wtconv/wtconv1d.py:23-31):
+ *   base_weight (C,1,K,K) | (C,1,K);  base_bias (C) or NULL;  base_scale C values;
+ *   wt_weight[l] (S*C,1,K,K) | (S*C,1,K) and wt_scale[l] S*C values, S = 4 (2-D) or 2 (1-D);
+ *   channel S*c+s of level l holds sub-band s (LL,LH,HL,HH | lo,hi) of input channel c
+ *   (fast_wtconv/cuda_haar/haar_cuda.py:13). */
+typedef struct wtconv_params {
+  const void* base_weight;
+  const void* base_bias;
+  const void* base_scale;
+  const void* wt_weight[WTCONV_MAX_LEVELS];
+  const void* wt_scale[WTCONV_MAX_LEVELS];
+} wtconv_params;
+
+/* Device pointers receiving the parameter gradients (float, same shapes as above).
+ * base_bias may be NULL when the layer has no bias. */
+typedef struct wtconv_param_grads {
+  float* base_weight;
+  float* base_bias;
+  float* base_scale;
+  float* wt_weight[WTCONV_MAX_LEVELS];
+  float* wt_scale[WTCONV_MAX_LEVELS];
+} wtconv_param_grads;
+
+/* ABI version of the loaded library (== WTCONV_ABI_VERSION). */
+int wtconv_abi_version(void);
+
+/* Message of the last failure on this thread ("" if none). */
+const char* wtconv_last_error(void);
+
+/* Largest odd kernel size the built kernels cover (cf. HAAR_MAX_K,
+ * fast_wtconv/cuda_haar/haar_common.cuh:32-49). */
+int wtconv_max_kernel_size(void);
+
+/* ------------------------------------------------------------------ 2-D layer
+ * Replaces, as one call each, what the reference composes from
+ * wavelet_2d_transform / wavelet_convs / wavelet_scale / inverse_2d_wavelet_transform /
+ * base_conv / base_scale (wtconv/wtconv2d.py:38-82) and, in the fast twin,
+ * fused_haar_conv_forward + ihaar_cascade + the cuDNN base conv
+ * (fast_wtconv/cuda_haar/haar_cuda.py:321-357,635-647).  Stride is not part of the
+ * kernels: the caller sub-samples the stride-1 result (wtconv2d.py:84-85). */
+size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass);
+
+int wtconv2d_forward(const void* x, void* out, const wtconv_params* params,
+                     int B, int C, int H, int W, int K, int levels,
+                     int dtype, int param_dtype,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* grad_x from grad_out: replaces autograd through wtconv2d.py:38-82 and
+ * WaveletBranchFunction.backward + conv2d_input (haar_cuda.py:359-413,650-656). */
+int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params,
+                            int B, int C, int H, int W, int K, int levels,
+                            int dtype, int param_dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Gradients of every trainable parameter (deterministic two-stage reduction; no
+ * atomics): replaces fused_haar_grad_weight + depthwise_grad_weight and the host
+ * algebra around them (haar_cuda.py:168-197,415-421,657-676). */
+int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+                             const wtconv_param_grads* grads,
+                             int B, int C, int H, int W, int K, int levels,
+                             int dtype, int param_dtype,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ 1-D layer
+ * Same three calls for wtconv/wtconv1d.py:38-82 (two sub-bands, 1/sqrt(2) butterflies). */
+size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass);
+
+int wtconv1d_forward(const void* x, void* out, const wtconv_params* params,
+                     int B, int C, int N, int K, int levels,
+                     int dtype, int param_dtype,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+int wtconv1d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params,
+                            int B, int C, int N, int K, int levels,
+                            int dtype, int param_dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+                             const wtconv_param_grads* grads,
+                             int B, int C, int N, int K, int levels,
+                             int dtype, int param_dtype,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WTCONV_HIP_H */

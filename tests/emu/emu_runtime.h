@@ -1,0 +1,97 @@
+// Host stand-in for the few HIP device facilities the WTConv kernels use, so that the
+// kernel sources can be compiled with g++ and run under AddressSanitizer without a GPU.
+// Test infrastructure only: a workgroup becomes a set of std::threads that meet at a
+// barrier for __syncthreads(); LDS becomes an exactly-sized heap block so that any
+// out-of-range LDS access is reported.
+#pragma once
+
+#include <barrier>
+#include <cmath>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <memory>
+#include <thread>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline
+#define __launch_bounds__(...)
+#define __align__(n)
+
+struct dim3 {
+  unsigned x, y, z;
+  dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+struct uint2 { uint32_t x, y; };
+struct alignas(16) uint4 { uint32_t x, y, z, w; };
+struct float2 { float x, y; };
+struct alignas(16) float4 { float x, y, z, w; };
+
+typedef void* hipStream_t;
+
+namespace emu {
+struct BlockState {
+  std::unique_ptr<std::barrier<>> bar;
+  float* lds = nullptr;
+  std::vector<float> xchg;
+  unsigned nthreads = 0;
+};
+inline thread_local BlockState* tls_block = nullptr;
+inline float* lds_base() { return tls_block->lds; }
+}  // namespace emu
+
+inline thread_local dim3 threadIdx, blockIdx, blockDim, gridDim;
+
+inline void __syncthreads() { emu::tls_block->bar->arrive_and_wait(); }
+
+inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+
+// Every thread of the block must call this the same number of times (true for the
+// kernels here: reductions sit outside divergent code).
+inline float __shfl_xor(float v, int mask, int /*width*/) {
+  emu::BlockState* b = emu::tls_block;
+  b->xchg[threadIdx.x] = v;
+  b->bar->arrive_and_wait();
+  const float r = b->xchg[threadIdx.x ^ static_cast<unsigned>(mask)];
+  b->bar->arrive_and_wait();
+  return r;
+}
+
+namespace emu {
+template <typename F>
+void launch(dim3 grid, dim3 block, size_t lds_bytes, F body) {
+  const unsigned nt = block.x * block.y * block.z;
+  for (unsigned bz = 0; bz < grid.z; ++bz)
+    for (unsigned by = 0; by < grid.y; ++by)
+      for (unsigned bx = 0; bx < grid.x; ++bx) {
+        BlockState st;
+        st.bar = std::make_unique<std::barrier<>>(nt);
+        st.nthreads = nt;
+        st.xchg.assign(nt, 0.f);
+        // exact size: ASan red zones catch LDS overruns; filled with NaN so that reads of
+        // never-written LDS show up in results
+        float* lds = lds_bytes ? static_cast<float*>(std::aligned_alloc(16, (lds_bytes + 15) / 16 * 16)) : nullptr;
+        for (size_t i = 0; i < lds_bytes / 4; ++i) lds[i] = std::nanf("");
+        st.lds = lds;
+        std::vector<std::thread> th;
+        th.reserve(nt);
+        for (unsigned t = 0; t < nt; ++t) {
+          th.emplace_back([&, t]() {
+            tls_block = &st;
+            threadIdx = dim3(t % block.x, (t / block.x) % block.y, t / (block.x * block.y));
+            blockIdx = dim3(bx, by, bz);
+            blockDim = block;
+            gridDim = grid;
+            body();
+          });
+        }
+        for (auto& x : th) x.join();
+        std::free(lds);
+      }
+}
+}  // namespace emu

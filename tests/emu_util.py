@@ -1,0 +1,81 @@
+"""Builds and drives the host emulation of the HIP kernels (tests/emu): the same kernel
+sources compiled with g++ -DWT_EMULATE under AddressSanitizer.  Test infrastructure."""
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EMU_DIR = os.path.join(ROOT, "tests", "emu")
+BUILD_DIR = os.path.join(EMU_DIR, "_build")
+EXE = os.path.join(BUILD_DIR, "emu_driver")
+SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(EMU_DIR, "emu_driver.cpp")]
+DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
+                  ("common.h", "kernels1d.h", "kernels2d.h", "plan.h")] + [
+    os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
+
+
+def build(force=False):
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    if not force and os.path.exists(EXE):
+        newest = max(os.path.getmtime(p) for p in DEPS)
+        if os.path.getmtime(EXE) >= newest:
+            return EXE
+    cmd = ["g++", "-std=c++20", "-O1", "-g", "-fsanitize=address,undefined",
+           "-fno-sanitize-recover=undefined", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
+           SOURCES[0], SOURCES[1], "-pthread", "-o", EXE]
+    subprocess.run(cmd, check=True, cwd=ROOT)
+    return EXE
+
+
+def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600):
+    """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays."""
+    exe = build()
+    if dims == 2:
+        B, C, H, W = x.shape
+        S, KK = 4, K * K
+    else:
+        B, C, W = x.shape
+        H = 1
+        S, KK = 2, K
+    L = len(wt_ws)
+    has_bias = base_b is not None
+    hdr = np.array([dims, B, C, H, W, K, L, dtype, pdtype, int(has_bias)], dtype=np.int32)
+    parts = [hdr.tobytes(), x.astype(np.float32).tobytes(), g.astype(np.float32).tobytes(),
+             base_w.astype(np.float32).tobytes()]
+    if has_bias:
+        parts.append(base_b.astype(np.float32).tobytes())
+    parts.append(base_s.astype(np.float32).tobytes())
+    for w, s in zip(wt_ws, wt_ss):
+        parts += [w.astype(np.float32).tobytes(), s.astype(np.float32).tobytes()]
+    with tempfile.TemporaryDirectory() as td:
+        fin, fout = os.path.join(td, "in.bin"), os.path.join(td, "out.bin")
+        with open(fin, "wb") as f:
+            f.write(b"".join(parts))
+        env = dict(os.environ)
+        env["ASAN_OPTIONS"] = "detect_leaks=0"
+        env.pop("LD_PRELOAD", None)
+        r = subprocess.run([exe, fin, fout], capture_output=True, text=True, timeout=timeout, env=env)
+        if r.returncode != 0:
+            raise RuntimeError(f"emu_driver failed ({r.returncode}):\n{r.stderr[-4000:]}")
+        raw = np.fromfile(fout, dtype=np.float32)
+    P = x.size
+    pos = 0
+
+    def take(n, shape):
+        nonlocal pos
+        a = raw[pos:pos + n].reshape(shape)
+        pos += n
+        return a
+
+    res = {"out": take(P, x.shape), "dx": take(P, x.shape), "dbase_w": take(C * KK, base_w.shape)}
+    if has_bias:
+        res["dbase_b"] = take(C, (C,))
+    res["dbase_s"] = take(C, base_s.shape)
+    res["dwt_ws"], res["dwt_ss"] = [], []
+    for w, s in zip(wt_ws, wt_ss):
+        res["dwt_ws"].append(take(w.size, w.shape))
+        res["dwt_ss"].append(take(s.size, s.shape))
+    assert pos == raw.size
+    return res

@@ -1,0 +1,115 @@
+"""Runs the HIP kernel sources on the host (g++ -DWT_EMULATE, AddressSanitizer + UBSan,
+one std::thread per GPU thread) through the same C ABI and checks them against the
+oracle.  This exercises the kernels' indexing, halo/padding/crop logic and reductions
+without a GPU; the arithmetic on the GPU itself is covered by the -m gpu tests."""
+import numpy as np
+import pytest
+import torch
+
+import emu_util
+from oracle import wtconv_ref as R
+
+
+def _bf16_round(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+def _case2d(B, C, H, W, K, L, bias, dtype=0, pdtype=0, seed=0):
+    rng = np.random.default_rng(seed)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    x, g = f(B, C, H, W), f(B, C, H, W)
+    bw, bb, bs = f(C, 1, K, K) * 0.3, (f(C) if bias else None), f(1, C, 1, 1)
+    ws = [f(4 * C, 1, K, K) * 0.3 for _ in range(L)]
+    ss = [f(1, 4 * C, 1, 1) for _ in range(L)]
+    if dtype:
+        x, g = _bf16_round(x), _bf16_round(g)
+    if pdtype:
+        bw, bs = _bf16_round(bw), _bf16_round(bs)
+        bb = _bf16_round(bb) if bias else None
+        ws, ss = [_bf16_round(w) for w in ws], [_bf16_round(s) for s in ss]
+    return x, g, bw, bb, bs, ws, ss
+
+
+def _oracle(dims, x, g, bw, bb, bs, ws, ss):
+    t = lambda a: torch.from_numpy(a).double().requires_grad_(True)
+    tx, tbw, tbs = t(x), t(bw), t(bs)
+    tbb = t(bb) if bb is not None else None
+    tws, tss = [t(w) for w in ws], [t(s) for s in ss]
+    fn = R.wtconv2d_ref if dims == 2 else R.wtconv1d_ref
+    out = fn(tx, tbw, tbb, tbs, tws, tss)
+    out.backward(torch.from_numpy(g).double())
+    res = {"out": out.detach().numpy(), "dx": tx.grad.numpy(), "dbase_w": tbw.grad.numpy(),
+           "dbase_s": tbs.grad.numpy(), "dwt_ws": [w.grad.numpy() for w in tws],
+           "dwt_ss": [s.grad.numpy() for s in tss]}
+    if bb is not None:
+        res["dbase_b"] = tbb.grad.numpy()
+    return res
+
+
+def _compare(got, want, rtol, atol_scale):
+    def chk(a, b, name):
+        scale = max(float(np.sqrt(np.mean(b.astype(np.float64) ** 2))), 1e-6)
+        np.testing.assert_allclose(a, b, rtol=rtol, atol=atol_scale * scale, err_msg=name)
+    for k in ("out", "dx", "dbase_w", "dbase_s"):
+        chk(got[k], want[k], k)
+    if "dbase_b" in want:
+        chk(got["dbase_b"], want["dbase_b"], "dbase_b")
+    for l, (a, b) in enumerate(zip(got["dwt_ws"], want["dwt_ws"])):
+        chk(a, b, f"dwt_w[{l}]")
+    for l, (a, b) in enumerate(zip(got["dwt_ss"], want["dwt_ss"])):
+        chk(a, b, f"dwt_s[{l}]")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _built():
+    emu_util.build()
+
+
+@pytest.mark.parametrize("B,C,H,W,K,L,bias", [
+    (2, 2, 8, 8, 3, 2, True),       # even sizes, 128-bit load path
+    (1, 2, 7, 7, 5, 2, True),       # odd at level 1 (7 -> 4 -> 2), scalar load path
+    (1, 1, 14, 14, 5, 2, False),    # odd at level 2, no bias
+    (1, 2, 9, 13, 3, 3, True),      # odd everywhere, H != W
+    (1, 1, 12, 20, 7, 1, True),     # K = 7, single level
+    (2, 1, 6, 10, 1, 2, True),      # K = 1 (no conv halo)
+    (1, 1, 28, 28, 5, 5, True),     # five levels: 28 14 7 4 2 1
+])
+def test_emulated_2d_fp32(B, C, H, W, K, L, bias):
+    x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, K)
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
+
+
+def test_emulated_2d_bf16_io_and_params():
+    x, g, bw, bb, bs, ws, ss = _case2d(1, 2, 8, 12, 5, 2, True, dtype=1, pdtype=1)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, 5, dtype=1, pdtype=1)
+    # inputs are bf16-exact, maths is fp32; only out/dx are rounded to bf16 on store
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=1e-2, atol_scale=1e-2)
+
+
+def test_emulated_2d_stage1_plane():
+    """One plane of the WTConvNeXt-T stage-1 shape (56x56, K=5, L=3)."""
+    x, g, bw, bb, bs, ws, ss = _case2d(1, 1, 56, 56, 5, 3, True)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, 5)
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
+
+
+def _case1d(B, C, N, K, L, bias, seed=0):
+    rng = np.random.default_rng(seed)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    return (f(B, C, N), f(B, C, N), f(C, 1, K) * 0.3, (f(C) if bias else None), f(1, C, 1),
+            [f(2 * C, 1, K) * 0.3 for _ in range(L)], [f(1, 2 * C, 1) for _ in range(L)])
+
+
+@pytest.mark.parametrize("B,C,N,K,L,bias", [
+    (2, 2, 64, 5, 3, True),
+    (1, 2, 37, 5, 3, True),        # odd lengths at several levels
+    (1, 1, 9, 3, 4, False),        # row shorter than 2^L
+    (1, 1, 2500, 5, 4, True),      # three tiles, ragged last tile
+    (1, 2, 100, 7, 2, True),
+    (1, 1, 40, 1, 2, True),
+])
+def test_emulated_1d_fp32(B, C, N, K, L, bias):
+    x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, bias)
+    got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K)
+    _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)

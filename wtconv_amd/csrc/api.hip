@@ -1,0 +1,410 @@
+// C ABI of libwtconv_hip.so (declared in include/wtconv_hip.h): argument checks, LDS
+// planning and kernel launches.  Nothing here allocates, frees or synchronises.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.h"
+#include "kernels1d.h"
+#include "kernels2d.h"
+#include "plan.h"
+
+namespace wt {
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#ifdef WT_EMULATE
+#define WT_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
+  ::emu::launch((grid), (block), (lds_bytes), [&]() { kernel(__VA_ARGS__); })
+static int check_launch(const char*) { return 0; }
+template <typename F> static int allow_lds(F, size_t) { return 0; }
+#else
+#define WT_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
+  hipLaunchKernelGGL(kernel, (grid), (block), (lds_bytes), (stream), __VA_ARGS__)
+static int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return 0;
+}
+// Workgroups above 64 KiB of dynamic LDS need the opt-in attribute.
+template <typename F> static int allow_lds(F kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return 0;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(bytes));
+  if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
+  return 0;
+}
+#endif
+
+static ParamTable to_table(const wtconv_params* p, int L) {
+  ParamTable t = {};
+  t.base_weight = p->base_weight;
+  t.base_bias = p->base_bias;
+  t.base_scale = p->base_scale;
+  for (int l = 0; l < L; ++l) { t.wt_weight[l] = p->wt_weight[l]; t.wt_scale[l] = p->wt_scale[l]; }
+  return t;
+}
+
+static int check_common(const char* fn, const wtconv_params* params, int B, int C, int K, int L,
+                        int dtype, int pdtype) {
+  if (B <= 0 || C <= 0) return fail(WTCONV_E_ARG, "%s: batch and channels must be positive (got %d, %d)", fn, B, C);
+  if (K < 1 || K % 2 == 0) return fail(WTCONV_E_ARG, "%s: kernel_size must be odd and positive (got %d)", fn, K);
+  if (K > wtconv_max_kernel_size())
+    return fail(WTCONV_E_UNSUPPORTED, "%s: kernel_size %d exceeds the largest built kernel (%d)", fn, K,
+                wtconv_max_kernel_size());
+  if (L < 1 || L > kMaxLevels) return fail(WTCONV_E_ARG, "%s: wt_levels must be 1-%d (got %d)", fn, kMaxLevels, L);
+  if (dtype != WTCONV_F32 && dtype != WTCONV_BF16) return fail(WTCONV_E_ARG, "%s: unknown dtype %d", fn, dtype);
+  if (pdtype != WTCONV_F32 && pdtype != WTCONV_BF16) return fail(WTCONV_E_ARG, "%s: unknown param dtype %d", fn, pdtype);
+  if (params == nullptr || params->base_weight == nullptr || params->base_scale == nullptr)
+    return fail(WTCONV_E_ARG, "%s: null parameter pointer", fn);
+  for (int l = 0; l < L; ++l)
+    if (params->wt_weight[l] == nullptr || params->wt_scale[l] == nullptr)
+      return fail(WTCONV_E_ARG, "%s: null parameter pointer at level %d", fn, l);
+  return 0;
+}
+
+static size_t fold_floats(int C, int S, int L, int KK) { return static_cast<size_t>(C) * (1 + S * L) * KK + C; }
+
+static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float* fb, int C, int S, int L,
+                       int KK, int flip, int use_bias, hipStream_t stream) {
+  const int total = C * (1 + S * L) * KK;
+  int blocks = (total + 255) / 256;
+  if (blocks > 1024) blocks = 1024;
+  WT_LAUNCH(fold_params_kernel, dim3(blocks), dim3(256), 0, stream, to_table(params, L), pdtype, fw, fb, C, S, L,
+            KK, flip, use_bias);
+  return check_launch("fold_params_kernel");
+}
+
+// ---- 2-D dispatch over (dtype, K) ---------------------------------------------------
+template <typename T, int K>
+static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl, int B,
+                       hipStream_t stream) {
+  auto kern = wt2d_plane_kernel<T, K, kTJ1, kTJC>;
+  const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
+  if (int e = allow_lds(kern, lds)) return e;
+  WT_LAUNCH(kern, dim3(B * pl.C), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
+  return check_launch("wt2d_plane_kernel");
+}
+
+template <typename T>
+static int run_plane2d_k(int K, const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
+                         int B, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_plane2d<T, 1>(x, out, fw, fb, pl, B, stream);
+    case 3: return run_plane2d<T, 3>(x, out, fw, fb, pl, B, stream);
+    case 5: return run_plane2d<T, 5>(x, out, fw, fb, pl, B, stream);
+    case 7: return run_plane2d<T, 7>(x, out, fw, fb, pl, B, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
+template <typename T, int K, int L>
+static int run_wgrad2d(const void* x, const void* g, float* partial, const Plan2D& pl, int B, int bchunk,
+                       int nchunk, hipStream_t stream) {
+  auto kern = wt2d_wgrad_kernel<T, K, L, kTJW>;
+  const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
+  if (int e = allow_lds(kern, lds)) return e;
+  WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(512), lds, stream, static_cast<const T*>(x), static_cast<const T*>(g),
+            partial, pl, B, bchunk);
+  return check_launch("wt2d_wgrad_kernel");
+}
+
+template <typename T, int K>
+static int run_wgrad2d_l(int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
+                         int bchunk, int nchunk, hipStream_t stream) {
+  switch (L) {
+    case 1: return run_wgrad2d<T, K, 1>(x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 2: return run_wgrad2d<T, K, 2>(x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 3: return run_wgrad2d<T, K, 3>(x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 4: return run_wgrad2d<T, K, 4>(x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 5: return run_wgrad2d<T, K, 5>(x, g, partial, pl, B, bchunk, nchunk, stream);
+  }
+  return fail(WTCONV_E_ARG, "wt_levels %d", L);
+}
+
+template <typename T>
+static int run_wgrad2d_k(int K, int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
+                         int bchunk, int nchunk, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_wgrad2d_l<T, 1>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 3: return run_wgrad2d_l<T, 3>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 5: return run_wgrad2d_l<T, 5>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 7: return run_wgrad2d_l<T, 7>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
+static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
+                        int H, int W, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes,
+                        void* stream_, int flip) {
+  if (int e = check_common(fn, params, B, C, K, L, dtype, pdtype)) return e;
+  if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
+  if (x == nullptr || out == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+  const Plan2D pl = make_plan2d(C, H, W, K, L, false, esz, x, out, nullptr);
+  if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
+    return fail(WTCONV_E_UNSUPPORTED,
+                "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
+                "plane-resident kernels", fn, H, W, L, static_cast<size_t>(pl.lds_floats) * 4, kLdsLimitBytes);
+  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  float* fw = static_cast<float*>(ws);
+  float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
+  if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
+  return dtype == WTCONV_F32 ? run_plane2d_k<float>(K, x, out, fw, fb, pl, B, stream)
+                             : run_plane2d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
+}
+
+// ---- 1-D dispatch -------------------------------------------------------------------
+template <typename T, int K>
+static int run_tile1d(const void* x, void* out, const float* fw, const float* fb, const Plan1D& pl, int B,
+                      hipStream_t stream) {
+  auto kern = wt1d_tile_kernel<T, K, kTJ1D>;
+  const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
+  if (int e = allow_lds(kern, lds)) return e;
+  WT_LAUNCH(kern, dim3(pl.ntiles, B * pl.C), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out),
+            fw, fb, pl);
+  return check_launch("wt1d_tile_kernel");
+}
+
+template <typename T>
+static int run_tile1d_k(int K, const void* x, void* out, const float* fw, const float* fb, const Plan1D& pl,
+                        int B, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_tile1d<T, 1>(x, out, fw, fb, pl, B, stream);
+    case 3: return run_tile1d<T, 3>(x, out, fw, fb, pl, B, stream);
+    case 5: return run_tile1d<T, 5>(x, out, fw, fb, pl, B, stream);
+    case 7: return run_tile1d<T, 7>(x, out, fw, fb, pl, B, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
+template <typename T, int K, int L>
+static int run_wgrad1d(const void* x, const void* g, float* partial, const Plan1D& pl, int B, int per_chunk,
+                       int nchunk, hipStream_t stream) {
+  auto kern = wt1d_wgrad_kernel<T, K, L, kTJ1D>;
+  const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
+  if (int e = allow_lds(kern, lds)) return e;
+  WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<const T*>(g),
+            partial, pl, B, per_chunk);
+  return check_launch("wt1d_wgrad_kernel");
+}
+
+template <typename T, int K>
+static int run_wgrad1d_l(int L, const void* x, const void* g, float* partial, const Plan1D& pl, int B,
+                         int per_chunk, int nchunk, hipStream_t stream) {
+  switch (L) {
+    case 1: return run_wgrad1d<T, K, 1>(x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 2: return run_wgrad1d<T, K, 2>(x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 3: return run_wgrad1d<T, K, 3>(x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 4: return run_wgrad1d<T, K, 4>(x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 5: return run_wgrad1d<T, K, 5>(x, g, partial, pl, B, per_chunk, nchunk, stream);
+  }
+  return fail(WTCONV_E_ARG, "wt_levels %d", L);
+}
+
+template <typename T>
+static int run_wgrad1d_k(int K, int L, const void* x, const void* g, float* partial, const Plan1D& pl, int B,
+                         int per_chunk, int nchunk, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_wgrad1d_l<T, 1>(L, x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 3: return run_wgrad1d_l<T, 3>(L, x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 5: return run_wgrad1d_l<T, 5>(L, x, g, partial, pl, B, per_chunk, nchunk, stream);
+    case 7: return run_wgrad1d_l<T, 7>(L, x, g, partial, pl, B, per_chunk, nchunk, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
+static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
+                       int N, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes, void* stream_,
+                       int flip) {
+  if (int e = check_common(fn, params, B, C, K, L, dtype, pdtype)) return e;
+  if (N <= 0) return fail(WTCONV_E_ARG, "%s: length must be positive (got %d)", fn, N);
+  if (x == nullptr || out == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+  if (static_cast<long long>(B) * C > 65535)
+    return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld exceeds the grid limit 65535", fn,
+                static_cast<long long>(B) * C);
+  const Plan1D pl = make_plan1d(C, N, K, L, false, esz, x, out, nullptr);
+  const size_t need = wtconv1d_workspace_bytes(B, C, N, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  float* fw = static_cast<float*>(ws);
+  float* fb = fw + static_cast<size_t>(C) * (1 + 2 * L) * K;
+  if (int e = launch_fold(params, pdtype, fw, fb, C, 2, L, K, flip, flip ? 0 : 1, stream)) return e;
+  return dtype == WTCONV_F32 ? run_tile1d_k<float>(K, x, out, fw, fb, pl, B, stream)
+                             : run_tile1d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
+}
+
+}  // namespace wt
+
+using namespace wt;
+
+extern "C" {
+
+int wtconv_abi_version(void) { return WTCONV_ABI_VERSION; }
+
+const char* wtconv_last_error(void) { return g_err; }
+
+int wtconv_max_kernel_size(void) { return 7; }
+
+size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
+  (void)H; (void)W;
+  if (B <= 0 || C <= 0 || K <= 0 || levels <= 0) return 0;
+  size_t floats;
+  if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
+    int bchunk, nchunk;
+    wgrad_chunks(B, C, &bchunk, &nchunk);
+    floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
+  } else {
+    floats = fold_floats(C, 4, levels, K * K);
+  }
+  return (floats * sizeof(float) + 255) / 256 * 256;
+}
+
+int wtconv2d_forward(const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W, int K,
+                     int levels, int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+  return plane2d_pass("wtconv2d_forward", x, out, params, B, C, H, W, K, levels, dtype, param_dtype, workspace,
+                      workspace_bytes, stream, 0);
+}
+
+int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params, int B, int C,
+                            int H, int W, int K, int levels, int dtype, int param_dtype, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+  return plane2d_pass("wtconv2d_backward_input", grad_out, grad_x, params, B, C, H, W, K, levels, dtype,
+                      param_dtype, workspace, workspace_bytes, stream, 1);
+}
+
+int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+                             const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels,
+                             int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
+                             void* stream_) {
+  const char* fn = "wtconv2d_backward_params";
+  const int L = levels;
+  if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
+  if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
+  if (x == nullptr || grad_out == nullptr || grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
+      (params->base_bias != nullptr && grads->base_bias == nullptr))
+    return fail(WTCONV_E_ARG, "%s: null gradient pointer", fn);
+  for (int l = 0; l < L; ++l)
+    if (grads->wt_weight[l] == nullptr || grads->wt_scale[l] == nullptr)
+      return fail(WTCONV_E_ARG, "%s: null gradient pointer at level %d", fn, l);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+  const Plan2D pl = make_plan2d(C, H, W, K, L, true, esz, x, grad_out, nullptr);
+  if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
+    return fail(WTCONV_E_UNSUPPORTED,
+                "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
+                "plane-resident kernels", fn, H, W, L, static_cast<size_t>(pl.lds_floats) * 4, kLdsLimitBytes);
+  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD_PARAMS);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  int bchunk, nchunk;
+  wgrad_chunks(B, C, &bchunk, &nchunk);
+  float* partial = static_cast<float*>(workspace);
+  const int e = dtype == WTCONV_F32
+                    ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+                    : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
+  if (e) return e;
+  GradTable gt = {};
+  gt.base_weight = grads->base_weight;
+  gt.base_bias = grads->base_bias;
+  gt.base_scale = grads->base_scale;
+  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
+  const int nthreads = C * (1 + 4 * L);
+  WT_LAUNCH(wgrad_finish_kernel, dim3((nthreads + 127) / 128), dim3(128), 0, stream, partial, nchunk,
+            to_table(params, L), param_dtype, gt, C, 4, L, K * K);
+  return check_launch("wgrad_finish_kernel");
+}
+
+size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass) {
+  if (B <= 0 || C <= 0 || N <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
+  size_t floats;
+  if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
+    const Plan1D pl = make_plan1d(C, N, K, levels, true, 4, nullptr, nullptr, nullptr);
+    int per_chunk, nchunk;
+    wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
+    floats = static_cast<size_t>(nchunk) * C * ((1 + 2 * levels) * K + 1);
+  } else {
+    floats = fold_floats(C, 2, levels, K);
+  }
+  return (floats * sizeof(float) + 255) / 256 * 256;
+}
+
+int wtconv1d_forward(const void* x, void* out, const wtconv_params* params, int B, int C, int N, int K,
+                     int levels, int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+  return tile1d_pass("wtconv1d_forward", x, out, params, B, C, N, K, levels, dtype, param_dtype, workspace,
+                     workspace_bytes, stream, 0);
+}
+
+int wtconv1d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params, int B, int C,
+                            int N, int K, int levels, int dtype, int param_dtype, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+  return tile1d_pass("wtconv1d_backward_input", grad_out, grad_x, params, B, C, N, K, levels, dtype,
+                     param_dtype, workspace, workspace_bytes, stream, 1);
+}
+
+int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+                             const wtconv_param_grads* grads, int B, int C, int N, int K, int levels,
+                             int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
+                             void* stream_) {
+  const char* fn = "wtconv1d_backward_params";
+  const int L = levels;
+  if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
+  if (N <= 0) return fail(WTCONV_E_ARG, "%s: length must be positive (got %d)", fn, N);
+  if (x == nullptr || grad_out == nullptr || grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
+      (params->base_bias != nullptr && grads->base_bias == nullptr))
+    return fail(WTCONV_E_ARG, "%s: null gradient pointer", fn);
+  for (int l = 0; l < L; ++l)
+    if (grads->wt_weight[l] == nullptr || grads->wt_scale[l] == nullptr)
+      return fail(WTCONV_E_ARG, "%s: null gradient pointer at level %d", fn, l);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+  const Plan1D pl = make_plan1d(C, N, K, L, true, esz, x, grad_out, nullptr);
+  const size_t need = wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_BACKWARD_PARAMS);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  int per_chunk, nchunk;
+  wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
+  if (nchunk > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
+  float* partial = static_cast<float*>(workspace);
+  const int e = dtype == WTCONV_F32
+                    ? run_wgrad1d_k<float>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream)
+                    : run_wgrad1d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream);
+  if (e) return e;
+  GradTable gt = {};
+  gt.base_weight = grads->base_weight;
+  gt.base_bias = grads->base_bias;
+  gt.base_scale = grads->base_scale;
+  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
+  const int nthreads = C * (1 + 2 * L);
+  WT_LAUNCH(wgrad_finish_kernel, dim3((nthreads + 127) / 128), dim3(128), 0, stream, partial, nchunk,
+            to_table(params, L), param_dtype, gt, C, 2, L, K);
+  return check_launch("wgrad_finish_kernel");
+}
+
+}  // extern "C"

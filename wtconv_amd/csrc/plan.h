@@ -1,0 +1,120 @@
+// Host-side planning: LDS layouts and launch geometry.  Pure C++, no device code.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "kernels1d.h"
+#include "kernels2d.h"
+
+namespace wt {
+
+inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// Strip widths of the 2-D kernels (outputs per work item along a row).
+constexpr int kTJ1 = 2;     // level 1 (2 x 2*TJ1 output pixels per item)
+constexpr int kTJC = 1;     // coarser levels
+constexpr int kTJW = 4;     // weight-gradient correlation strips
+
+// Fills the LDS layout of one plane.  with_grad_pyramid adds the padded pyramid of
+// grad_out used by the weight-gradient kernel (and drops the Z buffers it does not need).
+inline Plan2D make_plan2d(int C, int H, int W, int K, int L, bool with_grad_pyramid,
+                          size_t elem_size, const void* p0, const void* p1, const void* p2) {
+  Plan2D pl = {};
+  pl.C = C; pl.H = H; pl.W = W; pl.L = L;
+  const int R = K / 2;
+  pl.P = R > 1 ? R : 1;
+  pl.h[0] = H; pl.w[0] = W;
+  for (int l = 1; l <= L; ++l) { pl.h[l] = (pl.h[l - 1] + 1) / 2; pl.w[l] = (pl.w[l - 1] + 1) / 2; }
+  int off = 0;
+  for (int l = 0; l <= L; ++l) {
+    pl.astr[l] = pl.w[l] + 2 * pl.P;
+    pl.apl[l] = round_up(pl.astr[l] * (pl.h[l] + 2 * pl.P), 4);
+    pl.aoff[l] = off;
+    off += pl.apl[l] * (l == 0 ? 1 : 4);
+  }
+  if (!with_grad_pyramid) {
+    for (int l = 2; l <= L; ++l) {
+      pl.zstr[l] = pl.w[l - 1];
+      pl.zoff[l] = off;
+      off += round_up(pl.h[l - 1] * pl.w[l - 1], 4);
+    }
+  } else {
+    for (int l = 0; l <= L; ++l) {
+      pl.gstr[l] = pl.w[l] + kTJW;
+      pl.gpl[l] = round_up(pl.gstr[l] * (pl.h[l] + 1), 4);
+      pl.goff[l] = off;
+      off += pl.gpl[l] * (l == 0 ? 1 : 4);
+    }
+  }
+  pl.lds_floats = round_up(off + kLdsSlackFloats, 4);
+  const size_t plane_bytes = static_cast<size_t>(H) * W * elem_size;
+  auto aligned = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  pl.vec_ok = (plane_bytes % 16 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
+  pl.row_vec_ok = pl.vec_ok && (W % (2 * kTJ1) == 0);
+  return pl;
+}
+
+// Batch chunking of the weight-gradient kernels: enough workgroups to fill 256 CUs a few
+// times over, long enough chunks to amortise the end-of-chunk reduction.
+inline void wgrad_chunks(int B, int C, int* bchunk, int* nchunk) {
+  int want = (1536 + C - 1) / C;          // workgroups per channel
+  if (want < 1) want = 1;
+  if (want > B) want = B;
+  int bc = (B + want - 1) / want;
+  if (bc < 1) bc = 1;
+  *bchunk = bc;
+  *nchunk = (B + bc - 1) / bc;
+}
+
+// ---- 1-D ------------------------------------------------------------------------------
+constexpr int kTJ1D = 4;     // level coefficients per work item in the 1-D kernels
+constexpr int kTile1D = 1024;
+
+inline Plan1D make_plan1d(int C, int N, int K, int L, bool with_grad_pyramid, size_t elem_size,
+                          const void* p0, const void* p1, const void* p2) {
+  Plan1D pl = {};
+  pl.C = C; pl.N = N; pl.L = L;
+  const int R = K / 2;
+  const int gran = 1 << L;
+  int T = round_up(N, gran);
+  if (T > kTile1D) T = kTile1D;          // kTile1D is a multiple of 2^L for every L <= 5
+  pl.T = T;
+  pl.ntiles = (N + T - 1) / T;
+  int off = 0;
+  for (int l = 0; l <= L; ++l) {
+    pl.tl[l] = T >> l;
+    pl.hal[l] = R << (L - l);
+    pl.apl[l] = round_up(pl.tl[l] + 2 * pl.hal[l], 4);
+    pl.aoff[l] = off;
+    off += pl.apl[l] * (l == 0 ? 1 : 2);
+  }
+  if (!with_grad_pyramid) {
+    for (int l = 2; l <= L; ++l) { pl.zoff[l] = off; off += round_up(pl.tl[l - 1], 4); }
+  } else {
+    for (int l = 0; l <= L; ++l) {
+      pl.gpl[l] = round_up(pl.tl[l], kTJ1D) + kTJ1D;
+      pl.goff[l] = off;
+      off += pl.gpl[l] * (l == 0 ? 1 : 2);
+    }
+  }
+  pl.lds_floats = round_up(off + kLdsSlackFloats, 4);
+  const size_t row_bytes = static_cast<size_t>(N) * elem_size;
+  auto aligned = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  pl.vec_ok = (row_bytes % 16 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
+  return pl;
+}
+
+// (row, tile) pairs per workgroup of the 1-D weight-gradient kernel.
+inline void wgrad_chunks1d(int B, int C, int ntiles, int* per_chunk, int* nchunk) {
+  const int total = B * ntiles;
+  int want = (2048 + C - 1) / C;
+  if (want < 1) want = 1;
+  if (want > total) want = total;
+  int pc = (total + want - 1) / want;
+  if (pc < 1) pc = 1;
+  *per_chunk = pc;
+  *nchunk = (total + pc - 1) / pc;
+}
+
+}  // namespace wt
