@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the WTConv2d hot path on one MI355X.
+
+A step is one forward + backward (grad_x and every parameter gradient) of
+WTConv2d(96,96,kernel_size=5,wt_levels=3) on x[128,96,56,56] -- the WTConvNeXt-T stage-1
+shape -- through the module API, on synthetic N(0,1) tensors already resident in HBM.
+Prints ONE JSON line: images/s, the HBM roofline of the dominant kernel and of the whole
+step (algorithmic bytes 5*P*s per step, 2*P*s per kernel launch), and the CPU oracle timed
+on the host cores of the same box.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+VALU_PEAK_TFLOPS = 78.6         # fp32 vector FMA without packed-FP32 code generation
+
+WORKLOADS = {
+    # name: (C, H, W, K, L, batch)
+    "stage1": (96, 56, 56, 5, 3, 128),
+    "stage2": (192, 28, 28, 5, 3, 128),
+    "stage3": (384, 14, 14, 5, 2, 128),
+    "stage4": (768, 7, 7, 5, 2, 128),
+    "config1": (32, 64, 64, 5, 3, 8),
+}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--dtype", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="stage1")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary dtype and per-kernel timing")
+    ap.add_argument("--cpu-batch", type=int, default=16)
+    return ap.parse_args()
+
+
+def mac_per_pixel(K, L):
+    return K * K * (1.0 + sum(4.0 ** (1 - l) for l in range(1, L + 1)))
+
+
+def make_sets(torch, dev, dtype, C, H, W, B, nsets):
+    """nsets distinct (x, g) pairs so that successive steps do not hit the 256 MB
+    Infinity Cache with the same lines."""
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    sets = []
+    for _ in range(nsets):
+        x = torch.randn(B, C, H, W, generator=gen).to(device=dev, dtype=dtype)
+        g = torch.randn(B, C, H, W, generator=gen).to(device=dev, dtype=dtype)
+        sets.append((x.requires_grad_(True), g))
+    return sets
+
+
+def time_steps(torch, fn, nsets, steps, warmup):
+    for i in range(warmup):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        evs[i][0].record()
+        fn(i % nsets)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = [a.elapsed_time(b) for a, b in evs]         # ms, HIP events on the launch stream
+    return wall / steps * 1e3, statistics.median(per), min(per), sum(per) / len(per)
+
+
+def bench_layer(torch, dev, dtype_name, workload, steps, warmup, per_kernel=True):
+    import ctypes
+    import wtconv
+    from wtconv_amd import _lib
+    from wtconv_amd import functional as Fn
+    C, H, W, K, L, B = WORKLOADS[workload]
+    dtype = torch.float32 if dtype_name == "fp32" else torch.bfloat16
+    esz = 4 if dtype_name == "fp32" else 2
+    P = B * C * H * W
+    torch.manual_seed(0)
+    mod = wtconv.WTConv2d(C, C, K, wt_levels=L).to(dev)
+    if dtype_name == "bf16":
+        mod = mod.to(torch.bfloat16)
+    set_bytes = 3 * P * esz
+    nsets = max(3, int(600e6 // set_bytes) + 1)
+    sets = make_sets(torch, dev, dtype, C, H, W, B, nsets)
+
+    def step(i):
+        x, g = sets[i]
+        x.grad = None
+        for p in mod.parameters():
+            p.grad = None
+        out = mod(x)
+        out.backward(g)
+
+    wall_ms, med_ms, min_ms, avg_ms = time_steps(torch, step, nsets, steps, warmup)
+    res = {
+        "dtype": dtype_name, "workload": workload, "ms_per_step": wall_ms, "ms_per_step_events_median": med_ms,
+        "ms_per_step_events_min": min_ms, "images_per_s": B / (wall_ms * 1e-3),
+        "step_algorithmic_bytes": 5 * P * esz,
+        "step_GBps": 5 * P * esz / (wall_ms * 1e-3) / 1e9,
+        "step_frac_hbm": 5 * P * esz / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "step_GFLOP": 2 * 3 * mac_per_pixel(K, L) * P / 1e9,
+        "step_frac_valu": 2 * 3 * mac_per_pixel(K, L) * P / (wall_ms * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
+        "buffer_sets": nsets,
+    }
+    if not per_kernel:
+        return res
+
+    # per-entry-point timing through the C ABI (each call = parameter fold + one main kernel)
+    lib = _lib.load()
+    params = [mod.base_conv.weight, mod.base_conv.bias, mod.base_scale.weight,
+              [m.weight for m in mod.wavelet_convs], [m.weight for m in mod.wavelet_scale]]
+    pd, bw, bb, bs, ws, ss = Fn._prep_params(sets[0][0], *params)
+    tab = Fn._table(_lib.Params, bw, bb, bs, ws, ss)
+    f32 = lambda t: torch.empty(t.shape, dtype=torch.float32, device=dev)
+    gbufs = (f32(bw), f32(bb), f32(bs), [f32(w) for w in ws], [f32(s) for s in ss])
+    gtab = Fn._table(_lib.ParamGrads, *gbufs)
+    outs = [torch.empty_like(sets[i][0]) for i in range(nsets)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    dt, pdt = Fn._DT[dtype], Fn._DT[pd]
+    wsz = max(lib.wtconv2d_workspace_bytes(B, C, H, W, K, L, p) for p in (0, 1, 2))
+    wsp = torch.empty(wsz, dtype=torch.uint8, device=dev)
+    P_ = Fn._ptr
+
+    def k_fwd(i):
+        rc = lib.wtconv2d_forward(P_(sets[i][0]), P_(outs[i]), ctypes.byref(tab), B, C, H, W, K, L, dt, pdt,
+                                  P_(wsp), wsz, stream)
+        assert rc == 0, lib.wtconv_last_error()
+
+    def k_bwd_in(i):
+        rc = lib.wtconv2d_backward_input(P_(sets[i][1]), P_(outs[i]), ctypes.byref(tab), B, C, H, W, K, L, dt, pdt,
+                                         P_(wsp), wsz, stream)
+        assert rc == 0, lib.wtconv_last_error()
+
+    def k_bwd_par(i):
+        rc = lib.wtconv2d_backward_params(P_(sets[i][0]), P_(sets[i][1]), ctypes.byref(tab), ctypes.byref(gtab),
+                                          B, C, H, W, K, L, dt, pdt, P_(wsp), wsz, stream)
+        assert rc == 0, lib.wtconv_last_error()
+
+    kern = {}
+    for name, fn in (("wt2d_plane_kernel(forward)", k_fwd), ("wt2d_plane_kernel(backward_input)", k_bwd_in),
+                     ("wt2d_wgrad_kernel", k_bwd_par)):
+        _, med, mn, avg = time_steps(torch, fn, nsets, steps, warmup)
+        kern[name] = {"avg_ms": avg, "median_ms": med, "min_ms": mn,
+                      "algorithmic_bytes": 2 * P * esz,
+                      "GBps": 2 * P * esz / (avg * 1e-3) / 1e9}
+    res["kernels"] = kern
+    return res
+
+
+def cpu_baseline(torch, workload, cpu_batch):
+    """The CPU oracle (torch.nn.functional restatement of the reference layer) forward +
+    backward in fp32 on all host cores, on `cpu_batch` images of the same shape."""
+    from oracle import wtconv_ref as R
+    C, H, W, K, L, B = WORKLOADS[workload]
+    b = min(cpu_batch, B)
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    ref = R.RefWTConv2d(C, C, K, wt_levels=L)
+    x = torch.randn(b, C, H, W, requires_grad=True)
+    g = torch.randn(b, C, H, W)
+    times = []
+    t_start = time.perf_counter()
+    it = 0
+    while it < 2 + 5 or (time.perf_counter() - t_start < 10 and it < 60):
+        x.grad = None
+        for p in ref.parameters():
+            p.grad = None
+        t0 = time.perf_counter()
+        ref(x).backward(g)
+        dt = time.perf_counter() - t0
+        if it >= 2:
+            times.append(dt)
+        it += 1
+        if time.perf_counter() - t_start > 30:
+            break
+    med = statistics.median(times)
+    return {"value": b / med, "unit": "images/s", "cores": cores, "kind": "port",
+            "sample": f"{len(times)} timed fwd+bwd iterations (2 warm-ups) of the torch.nn.functional oracle, "
+                      f"fp32, batch {b} of the same {C}x{H}x{W} shape, torch threads={torch.get_num_threads()}",
+            "ms_per_iter": med * 1e3}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); the layer is data-parallel per "
+              "plane and no multi-GPU figure is produced", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    C, H, W, K, L, B = WORKLOADS[args.workload]
+
+    main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup,
+                           per_kernel=not args.no_extra)
+    line = {
+        "metric": "WTConv2d fwd+bwd images/s",
+        "value": main_res["images_per_s"],
+        "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.dtype == "fp32" else "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"WTConv2d({C},{C},kernel_size={K},wt_levels={L}) fwd+bwd on x[{B},{C},{H},{W}] "
+                               f"({args.workload}), all parameter grads, seeded default init"},
+        "step": {k: main_res[k] for k in ("step_algorithmic_bytes", "step_GBps", "step_frac_hbm", "step_GFLOP",
+                                          "step_frac_valu", "ms_per_step_events_median", "ms_per_step_events_min",
+                                          "buffer_sets")},
+    }
+    if "kernels" in main_res:
+        line["kernels"] = main_res["kernels"]
+        name, k = max(main_res["kernels"].items(), key=lambda kv: kv[1]["avg_ms"])
+        line["roofline"] = {"bound": "hbm", "kernel": name, "achieved": k["GBps"], "peak": HBM_PEAK_GBPS,
+                            "unit": "GB/s", "frac": k["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                            "avg_launch_ms": k["avg_ms"], "algorithmic_bytes_per_launch": k["algorithmic_bytes"]}
+    else:
+        line["roofline"] = {"bound": "hbm", "kernel": "whole step", "achieved": main_res["step_GBps"],
+                            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": main_res["step_frac_hbm"], "traffic": None}
+    if not args.no_extra:
+        other = "bf16" if args.dtype == "fp32" else "fp32"
+        o = bench_layer(torch, dev, other, args.workload, args.steps, args.warmup, per_kernel=False)
+        line["other_dtype"] = {k: o[k] for k in ("dtype", "ms_per_step", "images_per_s", "step_GBps", "step_frac_hbm")}
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch, args.workload, args.cpu_batch)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

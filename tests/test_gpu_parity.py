@@ -1,0 +1,208 @@
+"""GPU parity of the HIP WTConv layer against the CPU oracle, through the C ABI
+(ctypes -> libwtconv_hip.so).  Run with -m gpu on an MI355X."""
+import pytest
+import torch
+
+import parity_util as U
+from oracle import wtconv_ref as R
+
+pytestmark = pytest.mark.gpu
+
+
+def _mods():
+    import wtconv
+    from wtconv.wtconv1d import WTConv1d
+    return wtconv.WTConv2d, WTConv1d
+
+
+def _run_fp32(kind, C, K, L, shape, hip_device, bias=True, stride=1, seed=0):
+    W2, W1 = _mods()
+    ref, x, g = U.seeded_case(kind, C, K, L, shape, bias=bias, seed=seed, stride=stride)
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, K, L, stride=stride, bias=bias)
+    got = U.hip_run(mod, x, g, hip_device)
+    want = U.oracle_run(ref, x, g, torch.float64)
+    U.compare_all(got, want, U.assert_fp32)
+    return got, want
+
+
+# ------------------------------------------------------------------ 2-D, fp32
+def test_config1_forward_matches_cpu_reference_path(hip_device):
+    """WTConv2d(32,32,5,wt_levels=3), x[8,32,64,64], seed 0, default init, forward, against
+    the fp32 CPU run of the oracle (the reference's own CPU-runnable case)."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 32, 5, 3, (8, 32, 64, 64))
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 3).to(hip_device)
+    with torch.no_grad():
+        got = mod(x.to(hip_device)).cpu()
+        want32 = ref(x)
+        want64 = ref.double()(x.double())
+    torch.testing.assert_close(got, want32, rtol=U.FP32_RTOL, atol=U.FP32_ATOL)
+    torch.testing.assert_close(got.double(), want64, rtol=U.FP32_RTOL, atol=U.FP32_ATOL)
+    print(f"\nmax|hip-fp64| = {(got.double() - want64).abs().max():.3e}   "
+          f"max|cpu_fp32-fp64| = {(want32.double() - want64).abs().max():.3e}")
+
+
+def test_config1_forward_backward(hip_device):
+    _run_fp32("2d", 32, 5, 3, (8, 32, 64, 64), hip_device)
+
+
+@pytest.mark.parametrize("C,H,L", [(96, 56, 3), (192, 28, 3), (384, 14, 2), (768, 7, 2)])
+def test_stage_shapes_fp32_small_batch(hip_device, C, H, L):
+    """The four WTConvNeXt-T stage shapes (K=5) at batch 4; 28/14/7 exercise the in-kernel
+    odd-size padding at levels 3/2/1."""
+    _run_fp32("2d", C, 5, L, (4, C, H, H), hip_device)
+
+
+@pytest.mark.parametrize("shape,K,L,bias", [
+    ((3, 5, 9, 13), 3, 3, True),       # odd everywhere, H != W
+    ((2, 4, 7, 7), 5, 2, False),       # odd at level 1, no bias
+    ((2, 3, 12, 20), 7, 1, True),      # K = 7
+    ((2, 3, 6, 10), 1, 2, True),       # K = 1
+    ((1, 2, 28, 28), 5, 5, True),      # five levels (model stage-1/2 use 5 and 4)
+    ((2, 2, 56, 56), 5, 5, True),      # model stage 1: 56 28 14 7 4 2
+    ((1, 1, 1, 1), 3, 1, True),        # smallest plane
+    ((2, 3, 33, 17), 5, 4, True),
+])
+def test_edge_shapes_fp32(hip_device, shape, K, L, bias):
+    _run_fp32("2d", shape[1], K, L, shape, hip_device, bias=bias, seed=3)
+
+
+def test_stride_2d(hip_device):
+    _run_fp32("2d", 4, 3, 2, (2, 4, 11, 14), hip_device, stride=2)
+
+
+def test_fast_twin_matches_reference_naming_module(hip_device):
+    """fast_wtconv.wtconv_cuda.WTConv2d (fused-twin parameter names, positional order
+    kernel_size, stride, wt_levels, bias) gives the same result as wtconv.WTConv2d, and
+    draws the same default init under the same seed."""
+    from fast_wtconv.wtconv_cuda import WTConv2d as Fast
+    import wtconv
+    torch.manual_seed(0)
+    a = wtconv.WTConv2d(6, 6, 5, wt_levels=2)
+    torch.manual_seed(0)
+    b = Fast(6, 6, 5, 1, 2, True)
+    assert torch.equal(a.base_conv.weight, b.base_weight) and torch.equal(a.base_conv.bias, b.base_bias)
+    for i in range(2):
+        assert torch.equal(a.wavelet_convs[i].weight, b.wt_weights[i])
+        assert torch.equal(a.wavelet_scale[i].weight, b.wt_scales[i])
+    assert set(b.state_dict()) == {"base_weight", "base_scale", "base_bias", "wt_weights.0", "wt_weights.1",
+                                   "wt_scales.0", "wt_scales.1"}
+    x = torch.randn(2, 6, 10, 12, device=hip_device)
+    ya, yb = a.to(hip_device)(x), b.to(hip_device)(x)
+    assert torch.equal(ya, yb)
+
+
+# ------------------------------------------------------------------ 2-D, bf16
+@pytest.mark.parametrize("C,H,L", [(96, 56, 3), (192, 28, 3), (384, 14, 2), (768, 7, 2)])
+@pytest.mark.parametrize("bf16_params", [False, True])
+def test_stage_shapes_bf16_small_batch(hip_device, C, H, L, bf16_params):
+    """bf16 activations (and optionally bf16 parameters).  Oracle: fp32 reference maths on
+    the bf16-rounded inputs/parameters; tolerance 2e-2 relative."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", C, 5, L, (4, C, H, H))
+    U.randomize_scales(ref)
+    rb = lambda t: t.to(torch.bfloat16).float()
+    x, g = rb(x), rb(g)
+    if bf16_params:
+        with torch.no_grad():
+            for p in ref.parameters():
+                p.copy_(rb(p))
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, L)
+    got = U.hip_run(mod, x, g, hip_device, dtype=torch.bfloat16,
+                    param_dtype=torch.bfloat16 if bf16_params else None)
+    want = U.oracle_run(ref, x, g, torch.float32)
+    U.compare_all(got, want, U.assert_bf16)
+
+
+# ------------------------------------------------------------------ 1-D
+def test_config4_1d_small_batch(hip_device):
+    """WTConv1d(64,64,5,wt_levels=4) on rows of 4096 at batch 4."""
+    _run_fp32("1d", 64, 5, 4, (4, 64, 4096), hip_device)
+
+
+@pytest.mark.parametrize("shape,K,L,bias,stride", [
+    ((2, 3, 37), 5, 3, True, 1),
+    ((1, 2, 9), 3, 4, False, 1),
+    ((2, 2, 2500), 5, 4, True, 1),     # ragged last tile
+    ((1, 3, 1000), 7, 5, True, 1),
+    ((2, 2, 51), 3, 2, True, 2),       # stride = true average pool
+    ((1, 1, 1), 3, 1, True, 1),
+])
+def test_edge_shapes_1d(hip_device, shape, K, L, bias, stride):
+    _run_fp32("1d", shape[1], K, L, shape, hip_device, bias=bias, stride=stride, seed=5)
+
+
+def test_1d_bf16(hip_device):
+    _, W1 = _mods()
+    ref, x, g = U.seeded_case("1d", 16, 5, 4, (4, 16, 1024))
+    U.randomize_scales(ref)
+    rb = lambda t: t.to(torch.bfloat16).float()
+    x, g = rb(x), rb(g)
+    mod = U.copy_to_hip_module(ref, W1, "1d", 5, 4)
+    got = U.hip_run(mod, x, g, hip_device, dtype=torch.bfloat16)
+    want = U.oracle_run(ref, x, g, torch.float32)
+    U.compare_all(got, want, U.assert_bf16)
+
+
+# ------------------------------------------------------------------ full-size checks
+def test_config2_full_size_fp32(hip_device):
+    """WTConv2d(96,96,5,wt_levels=3) on x[128,96,56,56]: forward/input-gradient planes are
+    independent, so the first two samples are compared with the oracle run on just those;
+    the adjoint identity <f(x), g> = <x, f^T(g)> (bias removed) and linearity of the
+    parameter gradients in g are checked over the whole batch."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 96, 5, 3, (128, 96, 56, 56))
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 3).to(hip_device)
+    xd = x.to(hip_device).requires_grad_(True)
+    gd = g.to(hip_device)
+    out = mod(xd)
+    out.backward(gd)
+    torch.cuda.synchronize()
+    wo, wdx, _ = U.oracle_run(ref, x[:2], g[:2], torch.float64)
+    U.assert_fp32(out[:2].detach().cpu(), wo, "out[:2]")
+    U.assert_fp32(xd.grad[:2].cpu(), wdx, "grad_x[:2]")
+    # adjoint identity over the whole batch, in float64 on the device
+    bias_resp = (mod.base_scale.weight * mod.base_conv.bias.view(1, -1, 1, 1)).detach()
+    lhs = ((out.detach() - bias_resp).double() * gd.double()).sum()
+    rhs = (xd.detach().double() * xd.grad.double()).sum()
+    assert abs(lhs.item() - rhs.item()) <= 1e-6 * max(abs(lhs.item()), 1.0) + 1e-2
+    # parameter gradients: full batch equals the sum over two half batches (linearity),
+    # and the half-batch sums are compared with the fp64 oracle
+    full = {n: p.grad.clone() for n, p in mod.named_parameters() if p.grad is not None}
+    halves = []
+    for sl in (slice(0, 64), slice(64, 128)):
+        for p in mod.parameters():
+            p.grad = None
+        xs = x[sl].to(hip_device).requires_grad_(True)
+        mod(xs).backward(g[sl].to(hip_device))
+        halves.append({n: p.grad.clone() for n, p in mod.named_parameters() if p.grad is not None})
+    for n in full:
+        s = halves[0][n] + halves[1][n]
+        scale = full[n].abs().max().item()
+        assert (full[n] - s).abs().max().item() <= 2e-5 * scale + 1e-4, n
+
+
+def test_config2_full_size_param_grads_vs_oracle(hip_device):
+    """All parameter gradients of config 2 at the full batch against the fp64 oracle."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 96, 5, 3, (128, 96, 56, 56))
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 3)
+    _, _, gg = U.hip_run(mod, x, g, hip_device)
+    torch.set_num_threads(16)
+    _, _, wg = U.oracle_run(ref, x, g, torch.float64)
+    _, _, wg32 = U.oracle_run(ref, x, g, torch.float32)
+    # Each entry sums 128*56*56 = 401 408 products (|sum| up to a few thousand), so float32
+    # itself resolves these sums only to ~1e-7 of their magnitude: the absolute floor is
+    # 1e-6 of the tensor's largest entry (never below the stated 1e-4), rtol stays 1e-5.
+    for n, want in wg.items():
+        if n in ("wt_filter", "iwt_filter"):
+            continue
+        atol = max(U.FP32_ATOL, 1e-6 * want.abs().max().item())
+        torch.testing.assert_close(gg[n].double(), want, rtol=U.FP32_RTOL, atol=atol,
+                                   msg=lambda m, n=n: f"{n}: {m}")
+        e_hip = (gg[n].double() - want).abs().max().item()
+        e_cpu = (wg32[n].double() - want).abs().max().item()
+        print(f"\n{n}: max|hip-fp64| = {e_hip:.3e}, max|cpu_fp32-fp64| = {e_cpu:.3e}, max|want| = {want.abs().max():.1f}")
