@@ -331,9 +331,9 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   gt.base_bias = grads->base_bias;
   gt.base_scale = grads->base_scale;
   for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
-  const int nthreads = C * (1 + 4 * L);
-  WT_LAUNCH(wgrad_finish_kernel, dim3((nthreads + 127) / 128), dim3(128), 0, stream, partial, nchunk,
-            to_table(params, L), param_dtype, gt, C, 4, L, K * K);
+  const int nrec = (1 + 4 * L) * K * K + 1;
+  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(256), static_cast<size_t>(nrec) * sizeof(float),
+            stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 4, L, K * K);
   return check_launch("wgrad_finish_kernel");
 }
 
@@ -401,9 +401,9 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   gt.base_bias = grads->base_bias;
   gt.base_scale = grads->base_scale;
   for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
-  const int nthreads = C * (1 + 2 * L);
-  WT_LAUNCH(wgrad_finish_kernel, dim3((nthreads + 127) / 128), dim3(128), 0, stream, partial, nchunk,
-            to_table(params, L), param_dtype, gt, C, 2, L, K);
+  const int nrec = (1 + 2 * L) * K + 1;
+  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(256), static_cast<size_t>(nrec) * sizeof(float),
+            stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 2, L, K);
   return check_launch("wgrad_finish_kernel");
 }
 

@@ -130,16 +130,41 @@ __device__ __forceinline__ void analysis_level(const float* __restrict__ src, in
   }
 }
 
+// Load NR consecutive floats from LDS as vectors of VW floats (VW = 4: ds_read_b128,
+// VW = 2: ds_read_b64).  The address must be VW*4-byte aligned.
+template <int NR, int VW>
+__device__ __forceinline__ void lds_row(const float* __restrict__ a, float (&row)[NR]) {
+  static_assert(NR % VW == 0, "row length is padded to the vector width");
+  if constexpr (VW == 4) {
+#pragma unroll
+    for (int q = 0; q < NR / 4; ++q) {
+      const float4 v = reinterpret_cast<const float4*>(a)[q];
+      row[4 * q] = v.x; row[4 * q + 1] = v.y; row[4 * q + 2] = v.z; row[4 * q + 3] = v.w;
+    }
+  } else if constexpr (VW == 2) {
+#pragma unroll
+    for (int q = 0; q < NR / 2; ++q) {
+      const float2 v = reinterpret_cast<const float2*>(a)[q];
+      row[2 * q] = v.x; row[2 * q + 1] = v.y;
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < NR; ++q) row[q] = a[q];
+  }
+}
+
+constexpr int pad_to(int n, int m) { return (n + m - 1) / m * m; }
+
 // K x K correlation of TJ horizontally adjacent outputs; `a` points at the top-left input
-// of the first output's window.
-template <int K, int TJ>
+// of the first output's window (VW*4-byte aligned).
+template <int K, int TJ, int VW>
 __device__ __forceinline__ void conv_strip(const float* __restrict__ a, int astr,
                                            const float* __restrict__ wf, float (&y)[TJ]) {
+  constexpr int NR = pad_to(TJ + K - 1, VW);
 #pragma unroll
   for (int kh = 0; kh < K; ++kh) {
-    float row[TJ + K - 1];
-#pragma unroll
-    for (int q = 0; q < TJ + K - 1; ++q) row[q] = a[kh * astr + q];
+    float row[NR];
+    lds_row<NR, VW>(a + kh * astr, row);
 #pragma unroll
     for (int kw = 0; kw < K; ++kw) {
       const float wv = wf[kh * K + kw];
@@ -164,6 +189,7 @@ template <int K, int TJ>
 __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2D& pl, int l,
                                             const float* __restrict__ wl_f) {
   constexpr int R = K / 2;
+  constexpr int VW = (R >= 1) ? TJ : 1;   // window starts at column j0 when the halo equals R
   const int hl = pl.h[l], wl = pl.w[l];
   const int nstrip = (wl + TJ - 1) / TJ;
   const int items = hl * nstrip;
@@ -183,7 +209,7 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
     for (int s = 0; s < 4; ++s) {
 #pragma unroll
       for (int t = 0; t < TJ; ++t) y[s][t] = 0.f;
-      conv_strip<K, TJ>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, wl_f + s * K * K, y[s]);
+      conv_strip<K, TJ, VW>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, wl_f + s * K * K, y[s]);
     }
 #pragma unroll
     for (int t = 0; t < TJ; ++t) {
@@ -244,6 +270,8 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
                                             T* __restrict__ out_plane) {
   constexpr int R = K / 2;
   constexpr int NO = 2 * TJ;
+  constexpr int VW = (R >= 1) ? TJ : 1;
+  constexpr int VWX = (R >= 1) ? (NO >= 4 ? 4 : NO) : 1;
   const int hl = pl.h[1], wl = pl.w[1];
   const int nstrip = (wl + TJ - 1) / TJ;
   const int items = hl * nstrip;
@@ -263,7 +291,7 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
     for (int s = 0; s < 4; ++s) {
 #pragma unroll
       for (int t = 0; t < TJ; ++t) y[s][t] = 0.f;
-      conv_strip<K, TJ>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, w1_f + s * K * K, y[s]);
+      conv_strip<K, TJ, VW>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, w1_f + s * K * K, y[s]);
     }
     float o0[NO], o1[NO];
 #pragma unroll
@@ -279,9 +307,9 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
     const float* xw = X + (2 * i - R + P) * xstr + (2 * j0 - R + P);
 #pragma unroll
     for (int r = 0; r < K + 1; ++r) {
-      float row[NO + K - 1];
-#pragma unroll
-      for (int q = 0; q < NO + K - 1; ++q) row[q] = xw[r * xstr + q];
+      constexpr int NRX = pad_to(NO + K - 1, VWX);
+      float row[NRX];
+      lds_row<NRX, VWX>(xw + r * xstr, row);
       if (r < K) {
 #pragma unroll
         for (int kw = 0; kw < K; ++kw) {
@@ -358,17 +386,16 @@ __global__ __launch_bounds__(256) void wt2d_plane_kernel(const T* __restrict__ x
 // deterministic; the reference uses float atomics, fused_haar_conv.cu:331-341).
 //   dWt_l[c,s,kh,kw] = sum_{b,i,j} dY_l[s][i,j] * A_l[s][i+kh-R, j+kw-R]
 //   dWt_b[c,kh,kw]   = sum_{b,i,j} G[i,j] * x[i+kh-R, j+kw-R],   sumG[c] = sum G
-template <int K, int TJ>
+template <int K, int TJ, int VW>
 __device__ __forceinline__ void corr_strip(const float* __restrict__ a, int astr,
                                            const float* __restrict__ gy, float (&acc)[K * K]) {
+  constexpr int NR = pad_to(TJ + K - 1, VW);
   float dy[TJ];
-#pragma unroll
-  for (int t = 0; t < TJ; ++t) dy[t] = gy[t];
+  lds_row<TJ, (TJ % 4 == 0) ? 4 : 1>(gy, dy);
 #pragma unroll
   for (int kh = 0; kh < K; ++kh) {
-    float row[TJ + K - 1];
-#pragma unroll
-    for (int q = 0; q < TJ + K - 1; ++q) row[q] = a[kh * astr + q];
+    float row[NR];
+    lds_row<NR, VW>(a + kh * astr, row);
 #pragma unroll
     for (int kw = 0; kw < K; ++kw) {
 #pragma unroll
@@ -385,6 +412,7 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
   constexpr int KK = K * K;
   constexpr int R = K / 2;
   constexpr int NF = 1 + 4 * L;
+  constexpr int VW = (R >= 1 && TJ % 4 == 0) ? 4 : 1;
   const int c = blockIdx.x;
   const int chunk = blockIdx.y;
   const int tid = threadIdx.x;
@@ -431,7 +459,7 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
         const float* gy = G + i * pl.gstr[0] + j0;
 #pragma unroll
         for (int t = 0; t < TJ; ++t) gsum += gy[t];
-        corr_strip<K, TJ>(X + (i - R + P) * pl.astr[0] + (j0 - R + P), pl.astr[0], gy, accb);
+        corr_strip<K, TJ, VW>(X + (i - R + P) * pl.astr[0] + (j0 - R + P), pl.astr[0], gy, accb);
       }
     }
 #pragma unroll
@@ -443,7 +471,7 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
       for (int it = sub_tid; it < items; it += 2 * kWave) {
         const int i = it / nstrip;
         const int j0 = (it - i * nstrip) * TJ;
-        corr_strip<K, TJ>(A + (i - R + P) * pl.astr[l] + (j0 - R + P), pl.astr[l],
+        corr_strip<K, TJ, VW>(A + (i - R + P) * pl.astr[l] + (j0 - R + P), pl.astr[l],
                           G + i * pl.gstr[l] + j0, accl[l - 1]);
       }
     }
@@ -492,41 +520,49 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
 // Second stage: sum the per-chunk partials and apply the chain rule of the folding
 //   dw = gamma * dWt,  dgamma = sum_t w * dWt (+ bias * sumG for the base scale),
 //   dbias = gamma_b * sumG        (cf. fast_wtconv/cuda_haar/haar_cuda.py:168-197,657-676)
-// One thread per (channel, filter).  S = 4 (2-D) or 2 (1-D).
+// One workgroup per channel, one thread per (filter, tap); the per-filter dot products go
+// through LDS.  S = 4 (2-D) or 2 (1-D).  blockDim.x >= NF, dynamic LDS NF*KK floats.
 __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchunk, ParamTable p,
                                     int pdtype, GradTable gt, int C, int S, int L, int KK) {
+  WT_SHARED_FLOATS(prod);
   const int NF = 1 + S * L;
   const int stride = NF * KK + 1;
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= C * NF) return;
-  const int c = idx / NF, f = idx - c * NF;
-  float dot = 0.f;
-  if (f == 0) {
-    const float gam = load_param(p.base_scale, pdtype, c);
-    for (int t = 0; t < KK; ++t) {
-      float s = 0.f;
-      for (int ch = 0; ch < nchunk; ++ch) s += partial[(static_cast<size_t>(ch) * C + c) * stride + t];
-      gt.base_weight[c * KK + t] = gam * s;
-      dot = fmaf(load_param(p.base_weight, pdtype, c * KK + t), s, dot);
+  const int c = blockIdx.x;
+  for (int o = threadIdx.x; o < NF * KK; o += blockDim.x) {
+    float sum = 0.f;
+    for (int ch = 0; ch < nchunk; ++ch) sum += partial[(static_cast<size_t>(ch) * C + c) * stride + o];
+    const int f = o / KK, t = o - f * KK;
+    float gam, wv;
+    if (f == 0) {
+      gam = load_param(p.base_scale, pdtype, c);
+      wv = load_param(p.base_weight, pdtype, c * KK + t);
+      gt.base_weight[c * KK + t] = gam * sum;
+    } else {
+      const int l = (f - 1) / S, chn = c * S + (f - 1) % S;
+      gam = load_param(p.wt_scale[l], pdtype, chn);
+      wv = load_param(p.wt_weight[l], pdtype, chn * KK + t);
+      gt.wt_weight[l][chn * KK + t] = gam * sum;
     }
-    float sg = 0.f;
-    for (int ch = 0; ch < nchunk; ++ch) sg += partial[(static_cast<size_t>(ch) * C + c) * stride + NF * KK];
-    if (p.base_bias != nullptr) {
-      dot = fmaf(load_param(p.base_bias, pdtype, c), sg, dot);
-      if (gt.base_bias != nullptr) gt.base_bias[c] = gam * sg;
+    prod[o] = wv * sum;
+  }
+  const int o = threadIdx.x;
+  __syncthreads();
+  if (o < NF) {
+    float dot = 0.f;
+    for (int t = 0; t < KK; ++t) dot += prod[o * KK + t];
+    if (o == 0) {
+      // sumG sits in the last slot of the channel's partial record
+      float sg = 0.f;
+      for (int ch = 0; ch < nchunk; ++ch) sg += partial[(static_cast<size_t>(ch) * C + c) * stride + NF * KK];
+      if (p.base_bias != nullptr) {
+        dot = fmaf(load_param(p.base_bias, pdtype, c), sg, dot);
+        if (gt.base_bias != nullptr) gt.base_bias[c] = load_param(p.base_scale, pdtype, c) * sg;
+      }
+      gt.base_scale[c] = dot;
+    } else {
+      const int l = (o - 1) / S, chn = c * S + (o - 1) % S;
+      gt.wt_scale[l][chn] = dot;
     }
-    gt.base_scale[c] = dot;
-  } else {
-    const int l = (f - 1) / S, s_ = (f - 1) % S;
-    const int chn = c * S + s_;
-    const float gam = load_param(p.wt_scale[l], pdtype, chn);
-    for (int t = 0; t < KK; ++t) {
-      float s = 0.f;
-      for (int ch = 0; ch < nchunk; ++ch) s += partial[(static_cast<size_t>(ch) * C + c) * stride + f * KK + t];
-      gt.wt_weight[l][chn * KK + t] = gam * s;
-      dot = fmaf(load_param(p.wt_weight[l], pdtype, chn * KK + t), s, dot);
-    }
-    gt.wt_scale[l][chn] = dot;
   }
 }
 

@@ -12,8 +12,8 @@ namespace wt {
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Strip widths of the 2-D kernels (outputs per work item along a row).
-constexpr int kTJ1 = 2;     // level 1 (2 x 2*TJ1 output pixels per item)
-constexpr int kTJC = 1;     // coarser levels
+constexpr int kTJ1 = 4;     // level 1 (2 x 2*TJ1 output pixels per item)
+constexpr int kTJC = 2;     // coarser levels
 constexpr int kTJW = 4;     // weight-gradient correlation strips
 
 // Fills the LDS layout of one plane.  with_grad_pyramid adds the padded pyramid of
@@ -28,20 +28,20 @@ inline Plan2D make_plan2d(int C, int H, int W, int K, int L, bool with_grad_pyra
   for (int l = 1; l <= L; ++l) { pl.h[l] = (pl.h[l - 1] + 1) / 2; pl.w[l] = (pl.w[l - 1] + 1) / 2; }
   int off = 0;
   for (int l = 0; l <= L; ++l) {
-    pl.astr[l] = pl.w[l] + 2 * pl.P;
+    pl.astr[l] = round_up(pl.w[l] + 2 * pl.P, 4);
     pl.apl[l] = round_up(pl.astr[l] * (pl.h[l] + 2 * pl.P), 4);
     pl.aoff[l] = off;
     off += pl.apl[l] * (l == 0 ? 1 : 4);
   }
   if (!with_grad_pyramid) {
     for (int l = 2; l <= L; ++l) {
-      pl.zstr[l] = pl.w[l - 1];
+      pl.zstr[l] = round_up(pl.w[l - 1], 4);
       pl.zoff[l] = off;
-      off += round_up(pl.h[l - 1] * pl.w[l - 1], 4);
+      off += pl.zstr[l] * pl.h[l - 1];
     }
   } else {
     for (int l = 0; l <= L; ++l) {
-      pl.gstr[l] = pl.w[l] + kTJW;
+      pl.gstr[l] = round_up(pl.w[l] + 1, 4);
       pl.gpl[l] = round_up(pl.gstr[l] * (pl.h[l] + 1), 4);
       pl.goff[l] = off;
       off += pl.gpl[l] * (l == 0 ? 1 : 4);
