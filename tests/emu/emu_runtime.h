@@ -95,3 +95,5 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, F body) {
       }
 }
 }  // namespace emu
+
+inline int __clz(int v) { return v == 0 ? 32 : __builtin_clz(static_cast<unsigned>(v)); }

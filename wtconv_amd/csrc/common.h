@@ -17,8 +17,30 @@
 
 #ifdef WT_EMULATE
 #define WT_SHARED_FLOATS(name) float* name = ::emu::lds_base()
+#define WT_SCHED_FENCE() do {} while (0)
+#define WT_UNIFORM(x) (x)
+#define WT_CHUNK_FENCE() do {} while (0)
+#define WT_LAUNDER_UNIFORM_PTR(p) do {} while (0)
+typedef const float* wt_uniform_ptr;
 #else
+// Folded weights are read-only for the whole launch and indexed uniformly: the constant
+// address space makes the compiler fetch them with scalar loads into SGPRs even after a
+// barrier (global-address-space loads fall back to per-lane vector loads there).
+typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 #define WT_SHARED_FLOATS(name) extern __shared__ __align__(16) float name[]
+// nothing may be scheduled across this point (keeps LDS reads from being hoisted en masse)
+#define WT_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+// tells the compiler that an int is the same in every lane (keeps it in an SGPR, so that
+// everything indexed by it is fetched with scalar loads)
+#define WT_UNIFORM(x) __builtin_amdgcn_readfirstlane(x)
+// Compiler-level fence between the chunks of a work item: memory operations (the LDS row
+// reads of the next chunk) may not be moved above it, which bounds the live registers to
+// one chunk's rows.  Emits no instruction.
+#define WT_CHUNK_FENCE() do { asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0); } while (0)
+// Makes a uniform pointer opaque at this point, so that the scalar weight loads behind it
+// are issued here (25 SGPRs live) instead of being hoisted out of the row loop all at once
+// (hundreds of SGPRs, spilled to VGPR lanes).
+#define WT_LAUNDER_UNIFORM_PTR(p) asm volatile("" : "+s"(p))
 #endif
 
 namespace wt {
@@ -72,6 +94,19 @@ struct GradTable {
   float* wt_weight[kMaxLevels];
   float* wt_scale[kMaxLevels];
 };
+
+// Orders the computation of v[] before the next WT_CHUNK_FENCE (the fence alone only
+// orders memory operations; arithmetic would otherwise be sunk below it and every row read
+// of a work item would stay live at once).  Emits no instruction.
+template <int N>
+__device__ __forceinline__ void pin_values(float (&v)[N]) {
+#ifndef WT_EMULATE
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i]));
+#else
+  (void)v;
+#endif
+}
 
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {

@@ -34,8 +34,8 @@ struct Plan2D {
   int gstr[kMaxLevels + 1];    //   zero padded on the right/bottom, no halo
   int gpl[kMaxLevels + 1];
   int lds_floats;              // total, including slack
-  int vec_ok;                  // planes are 16-byte sized and aligned: 128-bit loads
-  int row_vec_ok;              // output row pieces may be stored as vectors
+  int vec_ok;                  // W % 4 == 0 and every tensor pointer aligned to 4 elements:
+                               //   rows can be moved as 4-element vectors
 };
 
 // ------------------------------------------------------------------ parameter folding
@@ -110,15 +110,88 @@ __device__ __forceinline__ void load_plane(const T* __restrict__ src, float* __r
   }
 }
 
+// Lane grouping without divisions: a level whose rows hold `nitem` work items is walked by
+// groups of GS = 2^gsh >= nitem consecutive lanes, one row per group and pass.  Lanes of a
+// group touch one LDS row at consecutive addresses.
+__device__ __forceinline__ int group_shift(int nitem) {
+  return nitem <= 1 ? 0 : 32 - __clz(nitem - 1);
+}
+
+// Four consecutive elements from HBM (address aligned to 4 elements).
+template <typename T>
+__device__ __forceinline__ void load4(const T* __restrict__ p, float (&v)[4]) {
+  if constexpr (sizeof(T) == 4) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  } else {
+    const uint2 q = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+  }
+}
+
+// Fused plane load + first analysis level for planes whose width is a multiple of 4:
+// a work item owns 2 input rows x 8 input columns (4 level-1 positions); it copies them
+// into the level-0 buffer and writes the four level-1 sub-bands, so the plane is read from
+// HBM with 16-byte (fp32) / 8-byte (bf16) loads and never re-read from LDS for level 1.
+// Odd H: the missing bottom row is the zero padding of wtconv2d.py:49-51.
+template <typename T>
+__device__ __forceinline__ void load_analysis1(const T* __restrict__ src, int H, int W,
+                                               float* __restrict__ d0, int str0, int P0,
+                                               float* __restrict__ d1, int str1, int pl1, int P1,
+                                               int tid, int nthreads) {
+  const int h1 = (H + 1) >> 1, w1 = W >> 1;
+  const int nstrip = (w1 + 3) >> 2;
+  const int gsh = group_shift(nstrip);
+  const int s = tid & ((1 << gsh) - 1);
+  if (s >= nstrip) return;
+  const int c0 = 8 * s;
+  for (int i = tid >> gsh; i < h1; i += nthreads >> gsh) {
+    float r0[8], r1[8];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int cc = c0 + 4 * hf;
+      float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+      if (cc < W) {
+        load4<T>(src + (2 * i) * W + cc, a);
+        if (2 * i + 1 < H) load4<T>(src + (2 * i + 1) * W + cc, b);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { r0[4 * hf + k] = a[k]; r1[4 * hf + k] = b[k]; }
+    }
+    float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+    float* o = d1 + (i + P1) * str1 + 4 * s + P1;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (c0 + k < W) {
+        x0[k] = r0[k];
+        if (2 * i + 1 < H) x0[str0 + k] = r1[k];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (4 * s + t < w1) {
+        const float a = r0[2 * t], b = r0[2 * t + 1], c = r1[2 * t], d = r1[2 * t + 1];
+        const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
+        o[t] = 0.5f * (sac + sbd);
+        o[pl1 + t] = 0.5f * (dac + dbd);
+        o[2 * pl1 + t] = 0.5f * (sac - sbd);
+        o[3 * pl1 + t] = 0.5f * (dac - dbd);
+      }
+    }
+  }
+}
+
 // One analysis level: src is the (haloed/padded, zero outside) LL plane of level l-1,
 // dst the four sub-band planes of level l.  Reading one past the source grid returns the
 // zero padding the reference applies to odd sizes (wtconv2d.py:49-51).
 __device__ __forceinline__ void analysis_level(const float* __restrict__ src, int sstr, int sP,
                                                float* __restrict__ dst, int dstr, int dpl, int dP,
                                                int hl, int wl, int tid, int nthreads) {
-  const int items = hl * wl;
-  for (int it = tid; it < items; it += nthreads) {
-    const int i = it / wl, j = it - i * wl;
+  const int gsh = group_shift(wl);
+  const int j = tid & ((1 << gsh) - 1);
+  if (j >= wl) return;
+  for (int i = tid >> gsh; i < hl; i += nthreads >> gsh) {
     const float* s0 = src + (2 * i + sP) * sstr + 2 * j + sP;
     const float a = s0[0], b = s0[1], c = s0[sstr], d = s0[sstr + 1];
     const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
@@ -157,9 +230,12 @@ constexpr int pad_to(int n, int m) { return (n + m - 1) / m * m; }
 
 // K x K correlation of TJ horizontally adjacent outputs; `a` points at the top-left input
 // of the first output's window (VW*4-byte aligned).
+// K x K correlation of TJ horizontally adjacent outputs; `a` points at the top-left input
+// of the first output's window (VW*4-byte aligned).  One call is one "chunk": its K row
+// reads are what the compiler may keep in flight at once.
 template <int K, int TJ, int VW>
 __device__ __forceinline__ void conv_strip(const float* __restrict__ a, int astr,
-                                           const float* __restrict__ wf, float (&y)[TJ]) {
+                                           wt_uniform_ptr wf, float (&y)[TJ]) {
   constexpr int NR = pad_to(TJ + K - 1, VW);
 #pragma unroll
   for (int kh = 0; kh < K; ++kh) {
@@ -171,6 +247,46 @@ __device__ __forceinline__ void conv_strip(const float* __restrict__ a, int astr
 #pragma unroll
       for (int t = 0; t < TJ; ++t) y[t] = fmaf(wv, row[t + kw], y[t]);
     }
+  }
+}
+
+// Adds sub-band s of one coefficient quad into the four reconstructed samples
+// (a b / c d), without the common factor 1/2: rows of the inverse Haar matrix.
+template <int S>
+__device__ __forceinline__ void ihaar_accumulate(float y, float& a, float& b, float& c, float& d) {
+  a += y;
+  if constexpr (S == 0) { b += y; c += y; d += y; }
+  if constexpr (S == 1) { b += y; c -= y; d -= y; }
+  if constexpr (S == 2) { b -= y; c += y; d -= y; }
+  if constexpr (S == 3) { b -= y; c -= y; d += y; }
+}
+
+// The four sub-band convolutions of TJ coefficient quads, accumulated straight into the
+// 2 x 2TJ reconstructed samples (scaled by 2), one fenced chunk per sub-band.
+template <int K, int TJ, int VW, int S>
+__device__ __forceinline__ void subband_chunks(const float* __restrict__ a, int astr, int apl,
+                                               wt_uniform_ptr wf, const float* __restrict__ zin,
+                                               float (&o0)[2 * TJ], float (&o1)[2 * TJ]) {
+  if constexpr (S < 4) {
+    float y[TJ];
+#pragma unroll
+    for (int t = 0; t < TJ; ++t) y[t] = 0.f;
+    wt_uniform_ptr w = wf + S * K * K;
+    WT_LAUNDER_UNIFORM_PTR(w);
+    conv_strip<K, TJ, VW>(a + S * apl, astr, w, y);
+    if constexpr (S == 0) {
+      if (zin != nullptr) {
+#pragma unroll
+        for (int t = 0; t < TJ; ++t) y[t] += zin[t];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TJ; ++t)
+      ihaar_accumulate<S>(y[t], o0[2 * t], o0[2 * t + 1], o1[2 * t], o1[2 * t + 1]);
+    pin_values(o0);
+    pin_values(o1);
+    WT_CHUNK_FENCE();
+    subband_chunks<K, TJ, VW, S + 1>(a, astr, apl, wf, zin, o0, o1);
   }
 }
 
@@ -187,12 +303,15 @@ __device__ __forceinline__ void ihaar4(float ll, float lh, float hl, float hh,
 // inverse Haar, cropped store into Z_l.
 template <int K, int TJ>
 __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2D& pl, int l,
-                                            const float* __restrict__ wl_f) {
+                                            wt_uniform_ptr wl_f) {
   constexpr int R = K / 2;
   constexpr int VW = (R >= 1) ? TJ : 1;   // window starts at column j0 when the halo equals R
   const int hl = pl.h[l], wl = pl.w[l];
   const int nstrip = (wl + TJ - 1) / TJ;
-  const int items = hl * nstrip;
+  const int gsh = group_shift(nstrip);
+  const int strip = threadIdx.x & ((1 << gsh) - 1);
+  if (strip >= nstrip) return;
+  const int j0 = strip * TJ;
   const int astr = pl.astr[l], apl = pl.apl[l], P = pl.P;
   const float* A = lds + pl.aoff[l];
   const bool has_carry = l < pl.L;
@@ -201,63 +320,47 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
   float* Zout = lds + pl.zoff[l];
   const int zout_str = pl.zstr[l];
   const int ho = pl.h[l - 1], wo = pl.w[l - 1];
-  for (int it = threadIdx.x; it < items; it += blockDim.x) {
-    const int i = it / nstrip;
-    const int j0 = (it - i * nstrip) * TJ;
-    float y[4][TJ];
+  for (int i = threadIdx.x >> gsh; i < hl; i += blockDim.x >> gsh) {
+    float o0[2 * TJ], o1[2 * TJ];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int t = 0; t < 2 * TJ; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
+    subband_chunks<K, TJ, VW, 0>(A + (i - R + P) * astr + (j0 - R + P), astr, apl, wl_f,
+                                 has_carry ? Zin + i * zin_str + j0 : nullptr, o0, o1);
+    const int r0 = 2 * i;
 #pragma unroll
-      for (int t = 0; t < TJ; ++t) y[s][t] = 0.f;
-      conv_strip<K, TJ, VW>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, wl_f + s * K * K, y[s]);
-    }
-#pragma unroll
-    for (int t = 0; t < TJ; ++t) {
-      const int j = j0 + t;
-      float ll = y[0][t];
-      if (has_carry) ll += Zin[i * zin_str + j];
-      float a, b, c, d;
-      ihaar4(ll, y[1][t], y[2][t], y[3][t], a, b, c, d);
-      const int r0 = 2 * i, c0 = 2 * j;
-      if (j < wl) {
-        if (c0 < wo) {
-          Zout[r0 * zout_str + c0] = a;
-          if (r0 + 1 < ho) Zout[(r0 + 1) * zout_str + c0] = c;
-        }
-        if (c0 + 1 < wo) {
-          Zout[r0 * zout_str + c0 + 1] = b;
-          if (r0 + 1 < ho) Zout[(r0 + 1) * zout_str + c0 + 1] = d;
-        }
+    for (int t = 0; t < 2 * TJ; ++t) {
+      const int c0 = 2 * j0 + t;
+      if (c0 < wo) {
+        Zout[r0 * zout_str + c0] = 0.5f * o0[t];
+        if (r0 + 1 < ho) Zout[(r0 + 1) * zout_str + c0] = 0.5f * o1[t];
       }
     }
   }
 }
 
+// Store up to N consecutive outputs (N multiple of 4, destination aligned to 4 elements
+// when vec4 is set); `nvalid` of them lie inside the row.
 template <typename T, int N>
-__device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[N], int nvalid, bool vec) {
-  if (vec && nvalid == N) {
-    if constexpr (sizeof(T) == 4) {
-      static_assert(N % 4 == 0, "row pieces are multiples of 4 elements");
+__device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[N], int nvalid, bool vec4) {
+  static_assert(N % 4 == 0, "row pieces are multiples of 4 elements");
 #pragma unroll
-      for (int k = 0; k < N / 4; ++k) {
+  for (int k = 0; k < N / 4; ++k) {
+    if (vec4 && 4 * k + 4 <= nvalid) {
+      if constexpr (sizeof(T) == 4) {
         float4 q;
         q.x = v[4 * k]; q.y = v[4 * k + 1]; q.z = v[4 * k + 2]; q.w = v[4 * k + 3];
-        reinterpret_cast<float4*>(dst)[k] = q;
-      }
-    } else {
-      static_assert(N % 4 == 0, "row pieces are multiples of 4 elements");
-#pragma unroll
-      for (int k = 0; k < N / 4; ++k) {
+        *reinterpret_cast<float4*>(dst + 4 * k) = q;
+      } else {
         uint2 q;
         q.x = static_cast<uint32_t>(f32_to_bf16(v[4 * k])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 1])) << 16);
         q.y = static_cast<uint32_t>(f32_to_bf16(v[4 * k + 2])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 3])) << 16);
-        reinterpret_cast<uint2*>(dst)[k] = q;
+        *reinterpret_cast<uint2*>(dst + 4 * k) = q;
       }
-    }
-  } else {
+    } else {
 #pragma unroll
-    for (int k = 0; k < N; ++k)
-      if (k < nvalid) dst[k] = from_f32<T>(v[k]);
+      for (int e = 4 * k; e < 4 * k + 4; ++e)
+        if (e < nvalid) dst[e] = from_f32<T>(v[e]);
+    }
   }
 }
 
@@ -265,8 +368,7 @@ __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[
 // (and bias) of the same 2 x 2TJ pixels, store to HBM.
 template <typename T, int K, int TJ>
 __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2D& pl,
-                                            const float* __restrict__ wb_f,
-                                            const float* __restrict__ w1_f, float bias,
+                                            wt_uniform_ptr wb_f, wt_uniform_ptr w1_f, float bias,
                                             T* __restrict__ out_plane) {
   constexpr int R = K / 2;
   constexpr int NO = 2 * TJ;
@@ -274,7 +376,10 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
   constexpr int VWX = (R >= 1) ? (NO >= 4 ? 4 : NO) : 1;
   const int hl = pl.h[1], wl = pl.w[1];
   const int nstrip = (wl + TJ - 1) / TJ;
-  const int items = hl * nstrip;
+  const int gsh = group_shift(nstrip);
+  const int strip = threadIdx.x & ((1 << gsh) - 1);
+  if (strip >= nstrip) return;
+  const int j0 = strip * TJ;
   const int astr = pl.astr[1], apl = pl.apl[1], P = pl.P;
   const float* A = lds + pl.aoff[1];
   const float* X = lds + pl.aoff[0];
@@ -283,58 +388,52 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
   const float* Zin = lds + pl.zoff[2];
   const int zin_str = pl.zstr[2];
   const int H = pl.H, W = pl.W;
-  for (int it = threadIdx.x; it < items; it += blockDim.x) {
-    const int i = it / nstrip;
-    const int j0 = (it - i * nstrip) * TJ;
-    float y[4][TJ];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-#pragma unroll
-      for (int t = 0; t < TJ; ++t) y[s][t] = 0.f;
-      conv_strip<K, TJ, VW>(A + s * apl + (i - R + P) * astr + (j0 - R + P), astr, w1_f + s * K * K, y[s]);
-    }
+  for (int i = threadIdx.x >> gsh; i < hl; i += blockDim.x >> gsh) {
     float o0[NO], o1[NO];
 #pragma unroll
-    for (int t = 0; t < TJ; ++t) {
-      float ll = y[0][t];
-      if (has_carry) ll += Zin[i * zin_str + j0 + t];
-      ihaar4(ll, y[1][t], y[2][t], y[3][t], o0[2 * t], o0[2 * t + 1], o1[2 * t], o1[2 * t + 1]);
-    }
-    // base conv of output rows 2i, 2i+1, columns 2j0 .. 2j0+NO-1
-    float b0[NO], b1[NO];
+    for (int t = 0; t < NO; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
+    subband_chunks<K, TJ, VW, 0>(A + (i - R + P) * astr + (j0 - R + P), astr, apl, w1_f,
+                                 has_carry ? Zin + i * zin_str + j0 : nullptr, o0, o1);
 #pragma unroll
-    for (int t = 0; t < NO; ++t) { b0[t] = bias; b1[t] = bias; }
+    for (int t = 0; t < NO; ++t) { o0[t] = fmaf(0.5f, o0[t], bias); o1[t] = fmaf(0.5f, o1[t], bias); }
+    // base conv of output rows 2i, 2i+1, columns 2j0 .. 2j0+NO-1, accumulated on top; input
+    // row r feeds output row 0 through kernel row r and output row 1 through kernel row r-1
     const float* xw = X + (2 * i - R + P) * xstr + (2 * j0 - R + P);
+    constexpr int NRX = pad_to(NO + K - 1, VWX);
+    wt_uniform_ptr wb = wb_f;
+    WT_LAUNDER_UNIFORM_PTR(wb);
 #pragma unroll
     for (int r = 0; r < K + 1; ++r) {
-      constexpr int NRX = pad_to(NO + K - 1, VWX);
       float row[NRX];
       lds_row<NRX, VWX>(xw + r * xstr, row);
       if (r < K) {
 #pragma unroll
         for (int kw = 0; kw < K; ++kw) {
-          const float wv = wb_f[r * K + kw];
+          const float wv = wb[r * K + kw];
 #pragma unroll
-          for (int t = 0; t < NO; ++t) b0[t] = fmaf(wv, row[t + kw], b0[t]);
+          for (int t = 0; t < NO; ++t) o0[t] = fmaf(wv, row[t + kw], o0[t]);
         }
       }
       if (r >= 1) {
 #pragma unroll
         for (int kw = 0; kw < K; ++kw) {
-          const float wv = wb_f[(r - 1) * K + kw];
+          const float wv = wb[(r - 1) * K + kw];
 #pragma unroll
-          for (int t = 0; t < NO; ++t) b1[t] = fmaf(wv, row[t + kw], b1[t]);
+          for (int t = 0; t < NO; ++t) o1[t] = fmaf(wv, row[t + kw], o1[t]);
         }
       }
+      if (r == K / 2) {
+        pin_values(o0);
+        pin_values(o1);
+        WT_CHUNK_FENCE();
+      }
     }
-#pragma unroll
-    for (int t = 0; t < NO; ++t) { o0[t] += b0[t]; o1[t] += b1[t]; }
     const int r0 = 2 * i, c0 = 2 * j0;
     int nvalid = W - c0;
     if (nvalid > NO) nvalid = NO;
     if (nvalid > 0) {
-      store_row<T, NO>(out_plane + r0 * W + c0, o0, nvalid, pl.row_vec_ok != 0);
-      if (r0 + 1 < H) store_row<T, NO>(out_plane + (r0 + 1) * W + c0, o1, nvalid, pl.row_vec_ok != 0);
+      store_row<T, NO>(out_plane + r0 * W + c0, o0, nvalid, pl.vec_ok != 0);
+      if (r0 + 1 < H) store_row<T, NO>(out_plane + (r0 + 1) * W + c0, o1, nvalid, pl.vec_ok != 0);
     }
   }
 }
@@ -358,20 +457,29 @@ __global__ __launch_bounds__(256) void wt2d_plane_kernel(const T* __restrict__ x
   const int plane = blockIdx.x;
   const int c = plane % pl.C;
   const int NF = 1 + 4 * pl.L;
-  const float* fwc = fw + static_cast<size_t>(c) * NF * KK;
+  wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
   const size_t plane_off = static_cast<size_t>(plane) * pl.H * pl.W;
 
   zero_lds(lds, pl.lds_floats);
   __syncthreads();
-  load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, pl.vec_ok != 0);
+  int l0 = 1;
+  if (pl.vec_ok) {
+    load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
+                      lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, threadIdx.x, blockDim.x);
+    l0 = 2;
+  } else {
+    load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, false);
+  }
   __syncthreads();
-  for (int l = 1; l <= pl.L; ++l) {
+  for (int lv = l0; lv <= pl.L; ++lv) {
+    const int l = WT_UNIFORM(lv);
     const float* src = lds + pl.aoff[l - 1];   // sub-band 0 (or the input plane)
     analysis_level(src, pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
                    pl.h[l], pl.w[l], threadIdx.x, blockDim.x);
     __syncthreads();
   }
-  for (int l = pl.L; l >= 2; --l) {
+  for (int lv = pl.L; lv >= 2; --lv) {
+    const int l = WT_UNIFORM(lv);
     synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK);
     __syncthreads();
   }
@@ -402,6 +510,8 @@ __device__ __forceinline__ void corr_strip(const float* __restrict__ a, int astr
       for (int t = 0; t < TJ; ++t) acc[kh * K + kw] = fmaf(dy[t], row[t + kw], acc[kh * K + kw]);
     }
   }
+  pin_values(acc);
+  WT_CHUNK_FENCE();
 }
 
 template <typename T, int K, int L, int TJ>
@@ -435,13 +545,23 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
   __syncthreads();
 
   const int b_end = (chunk + 1) * bchunk < B ? (chunk + 1) * bchunk : B;
-  for (int b = chunk * bchunk; b < b_end; ++b) {
+  for (int bv = chunk * bchunk; bv < b_end; ++bv) {
+    const int b = WT_UNIFORM(bv);
     const size_t plane_off = (static_cast<size_t>(b) * pl.C + c) * pl.H * pl.W;
-    load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, pl.vec_ok != 0);
-    load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, pl.vec_ok != 0);
+    int l0 = 1;
+    if (pl.vec_ok) {
+      load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], P,
+                        lds + pl.aoff[1], pl.astr[1], pl.apl[1], P, tid, blockDim.x);
+      load_analysis1<T>(g + plane_off, pl.H, pl.W, lds + pl.goff[0], pl.gstr[0], 0,
+                        lds + pl.goff[1], pl.gstr[1], pl.gpl[1], 0, tid, blockDim.x);
+      l0 = 2;
+    } else {
+      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, false);
+      load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, false);
+    }
     __syncthreads();
-#pragma unroll
-    for (int l = 1; l <= L; ++l) {
+    for (int lv = l0; lv <= L; ++lv) {
+      const int l = WT_UNIFORM(lv);
       analysis_level(lds + pl.aoff[l - 1], pl.astr[l - 1], P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], P,
                      pl.h[l], pl.w[l], tid, blockDim.x);
       analysis_level(lds + pl.goff[l - 1], pl.gstr[l - 1], 0, lds + pl.goff[l], pl.gstr[l], pl.gpl[l], 0,
@@ -450,29 +570,41 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
     }
     {  // base conv: all threads share the full-resolution plane
       const int nstrip = (pl.W + TJ - 1) / TJ;
-      const int items = pl.H * nstrip;
-      const float* X = lds + pl.aoff[0];
-      const float* G = lds + pl.goff[0];
-      for (int it = tid; it < items; it += blockDim.x) {
-        const int i = it / nstrip;
-        const int j0 = (it - i * nstrip) * TJ;
-        const float* gy = G + i * pl.gstr[0] + j0;
+      const int gsh = group_shift(nstrip);
+      const int strip = tid & ((1 << gsh) - 1);
+      if (strip < nstrip) {
+        const int j0 = strip * TJ;
+        const float* X = lds + pl.aoff[0] + (j0 - R + P);
+        const float* G = lds + pl.goff[0] + j0;
+        for (int i = tid >> gsh; i < pl.H; i += blockDim.x >> gsh) {
+          const float* gy = G + i * pl.gstr[0];
 #pragma unroll
-        for (int t = 0; t < TJ; ++t) gsum += gy[t];
-        corr_strip<K, TJ, VW>(X + (i - R + P) * pl.astr[0] + (j0 - R + P), pl.astr[0], gy, accb);
+          for (int t = 0; t < TJ; ++t) gsum += gy[t];
+          corr_strip<K, TJ, VW>(X + (i - R + P) * pl.astr[0], pl.astr[0], gy, accb);
+        }
+      }
+    }
+    {  // level 1: strips of TJ; the two waves of a sub-band share its rows
+      const int nstrip = (pl.w[1] + TJ - 1) / TJ;
+      const int gsh = group_shift(nstrip);
+      const int strip = sub_tid & ((1 << gsh) - 1);
+      if (strip < nstrip) {
+        const int j0 = strip * TJ;
+        const float* A = lds + pl.aoff[1] + sb * pl.apl[1] + (j0 - R + P);
+        const float* G = lds + pl.goff[1] + sb * pl.gpl[1] + j0;
+        for (int i = sub_tid >> gsh; i < pl.h[1]; i += (2 * kWave) >> gsh)
+          corr_strip<K, TJ, VW>(A + (i - R + P) * pl.astr[1], pl.astr[1], G + i * pl.gstr[1], accl[0]);
       }
     }
 #pragma unroll
-    for (int l = 1; l <= L; ++l) {
-      const int nstrip = (pl.w[l] + TJ - 1) / TJ;
-      const int items = pl.h[l] * nstrip;
-      const float* A = lds + pl.aoff[l] + sb * pl.apl[l];
-      const float* G = lds + pl.goff[l] + sb * pl.gpl[l];
-      for (int it = sub_tid; it < items; it += 2 * kWave) {
-        const int i = it / nstrip;
-        const int j0 = (it - i * nstrip) * TJ;
-        corr_strip<K, TJ, VW>(A + (i - R + P) * pl.astr[l] + (j0 - R + P), pl.astr[l],
-                          G + i * pl.gstr[l] + j0, accl[l - 1]);
+    for (int l = 2; l <= L; ++l) {   // coarse levels: one coefficient per item keeps the lanes busy
+      const int gsh = group_shift(pl.w[l]);
+      const int j0 = sub_tid & ((1 << gsh) - 1);
+      if (j0 < pl.w[l]) {
+        const float* A = lds + pl.aoff[l] + sb * pl.apl[l] + (j0 - R + P);
+        const float* G = lds + pl.goff[l] + sb * pl.gpl[l] + j0;
+        for (int i = sub_tid >> gsh; i < pl.h[l]; i += (2 * kWave) >> gsh)
+          corr_strip<K, 1, 1>(A + (i - R + P) * pl.astr[l], pl.astr[l], G + i * pl.gstr[l], accl[l - 1]);
       }
     }
     __syncthreads();

@@ -48,10 +48,9 @@ inline Plan2D make_plan2d(int C, int H, int W, int K, int L, bool with_grad_pyra
     }
   }
   pl.lds_floats = round_up(off + kLdsSlackFloats, 4);
-  const size_t plane_bytes = static_cast<size_t>(H) * W * elem_size;
-  auto aligned = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-  pl.vec_ok = (plane_bytes % 16 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
-  pl.row_vec_ok = pl.vec_ok && (W % (2 * kTJ1) == 0);
+  const uintptr_t mask = 4 * elem_size - 1;       // 4-element vectors: 16 B (fp32) / 8 B (bf16)
+  auto aligned = [mask](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
+  pl.vec_ok = (W % 4 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
   return pl;
 }
 
