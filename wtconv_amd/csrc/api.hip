@@ -45,6 +45,24 @@ template <typename F> static int allow_lds(F kernel, size_t bytes) {
 }
 #endif
 
+// Compute units of the current device (cached per thread; 256 on MI355X).
+static int compute_units() {
+#ifdef WT_EMULATE
+  return 2;
+#else
+  static thread_local int cached_dev = -1, cached_cu = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != cached_dev) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached_dev = dev;
+    cached_cu = n;
+  }
+  return cached_cu;
+#endif
+}
+
 static ParamTable to_table(const wtconv_params* p, int L) {
   ParamTable t = {};
   t.base_weight = p->base_weight;
@@ -91,7 +109,9 @@ static int run_plane2d(const void* x, void* out, const float* fw, const float* f
   auto kern = wt2d_plane_kernel<T, K, kTJ1, kTJC>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
-  WT_LAUNCH(kern, dim3(B * pl.C), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
+  int nwg = resident_workgroups(compute_units(), lds, 4, 8);
+  if (nwg > B * pl.C) nwg = B * pl.C;
+  WT_LAUNCH(kern, dim3(nwg), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
 }
 
@@ -152,7 +172,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  const Plan2D pl = make_plan2d(C, H, W, K, L, false, esz, x, out, nullptr);
+  const Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
   if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
     return fail(WTCONV_E_UNSUPPORTED,
                 "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
@@ -264,6 +284,21 @@ const char* wtconv_last_error(void) { return g_err; }
 
 int wtconv_max_kernel_size(void) { return 7; }
 
+#if defined(WT_PHASE_TIMING) && !defined(WT_EMULATE)
+// Profiling aid, only in -DWT_PHASE_TIMING builds: copies (and optionally clears) the 16
+// per-phase tick counters.  Synchronises the device.
+int wtconv_debug_phase_ticks(unsigned long long* out16, int reset) {
+  if (hipDeviceSynchronize() != hipSuccess) return WTCONV_E_LAUNCH;
+  if (out16 && hipMemcpyFromSymbol(out16, HIP_SYMBOL(wt_phase_ticks), 16 * sizeof(unsigned long long)) != hipSuccess)
+    return WTCONV_E_LAUNCH;
+  if (reset) {
+    unsigned long long z[16] = {0};
+    if (hipMemcpyToSymbol(HIP_SYMBOL(wt_phase_ticks), z, sizeof(z)) != hipSuccess) return WTCONV_E_LAUNCH;
+  }
+  return 0;
+}
+#endif
+
 size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
   (void)H; (void)W;
   if (B <= 0 || C <= 0 || K <= 0 || levels <= 0) return 0;
@@ -310,7 +345,7 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  const Plan2D pl = make_plan2d(C, H, W, K, L, true, esz, x, grad_out, nullptr);
+  const Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr);
   if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
     return fail(WTCONV_E_UNSUPPORTED,
                 "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "

@@ -19,6 +19,8 @@
 #define WT_SHARED_FLOATS(name) float* name = ::emu::lds_base()
 #define WT_SCHED_FENCE() do {} while (0)
 #define WT_UNIFORM(x) (x)
+#define WT_LDS_BARRIER() __syncthreads()
+#define WT_WAIT_VMEM() do {} while (0)
 #define WT_CHUNK_FENCE() do {} while (0)
 #define WT_LAUNDER_UNIFORM_PTR(p) do {} while (0)
 typedef const float* wt_uniform_ptr;
@@ -33,6 +35,19 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 // tells the compiler that an int is the same in every lane (keeps it in an SGPR, so that
 // everything indexed by it is fetched with scalar loads)
 #define WT_UNIFORM(x) __builtin_amdgcn_readfirstlane(x)
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for
+// every outstanding HBM load, i.e. for the prefetch of the next plane issued just before.
+#define WT_LDS_BARRIER()                                                \
+  do {                                                                  \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");     \
+    __builtin_amdgcn_s_barrier();                                       \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");     \
+  } while (0)
+// s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt left at their maxima).
+// gfx950 counts loads and stores in the same counter; waiting for the prefetch loads
+// *before* the output stores are issued lets those stores drain in the background instead
+// of being waited for at the top of the next plane.
+#define WT_WAIT_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)
 // Compiler-level fence between the chunks of a work item: memory operations (the LDS row
 // reads of the next chunk) may not be moved above it, which bounds the live registers to
 // one chunk's rows.  Emits no instruction.
@@ -41,6 +56,25 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 // are issued here (25 SGPRs live) instead of being hoisted out of the row loop all at once
 // (hundreds of SGPRs, spilled to VGPR lanes).
 #define WT_LAUNDER_UNIFORM_PTR(p) asm volatile("" : "+s"(p))
+#endif
+
+// Optional profiling aid (off in the product build): -DWT_PHASE_TIMING makes wave 0 of
+// every workgroup add the shader-clock ticks it spent in each kernel phase to
+// wt_phase_ticks[], readable through wtconv_debug_phase_ticks().
+#if defined(WT_PHASE_TIMING) && !defined(WT_EMULATE)
+__device__ unsigned long long wt_phase_ticks[16];
+#define WT_TICK_INIT() long long wt_t_prev = clock64()
+#define WT_TICK(k)                                                                         \
+  do {                                                                                     \
+    if (threadIdx.x == 0) {                                                                \
+      const long long wt_t_now = clock64();                                                \
+      atomicAdd(&wt_phase_ticks[k], static_cast<unsigned long long>(wt_t_now - wt_t_prev)); \
+      wt_t_prev = wt_t_now;                                                                \
+    }                                                                                      \
+  } while (0)
+#else
+#define WT_TICK_INIT() do {} while (0)
+#define WT_TICK(k) do {} while (0)
 #endif
 
 namespace wt {

@@ -19,6 +19,8 @@
 
 namespace wt {
 
+constexpr int kFetchPasses = 2;  // 2x4 pieces of the next plane a thread may hold in registers
+
 // LDS layout of one plane, computed on the host (plan.h).
 struct Plan2D {
   int C, H, W, L;
@@ -36,6 +38,9 @@ struct Plan2D {
   int lds_floats;              // total, including slack
   int vec_ok;                  // W % 4 == 0 and every tensor pointer aligned to 4 elements:
                                //   rows can be moved as 4-element vectors
+  int prefetch;                // vec_ok and a plane is at most kFetchPasses pieces per thread:
+                               //   the next plane is fetched into registers during compute
+  int nplanes;                 // B * C
 };
 
 // ------------------------------------------------------------------ parameter folding
@@ -131,7 +136,7 @@ __device__ __forceinline__ void load4(const T* __restrict__ p, float (&v)[4]) {
 }
 
 // Fused plane load + first analysis level for planes whose width is a multiple of 4:
-// a work item owns 2 input rows x 8 input columns (4 level-1 positions); it copies them
+// a work item owns 2 input rows x 4 input columns (2 level-1 positions); it copies them
 // into the level-0 buffer and writes the four level-1 sub-bands, so the plane is read from
 // HBM with 16-byte (fp32) / 8-byte (bf16) loads and never re-read from LDS for level 1.
 // Odd H: the missing bottom row is the zero padding of wtconv2d.py:49-51.
@@ -140,39 +145,91 @@ __device__ __forceinline__ void load_analysis1(const T* __restrict__ src, int H,
                                                float* __restrict__ d0, int str0, int P0,
                                                float* __restrict__ d1, int str1, int pl1, int P1,
                                                int tid, int nthreads) {
-  const int h1 = (H + 1) >> 1, w1 = W >> 1;
-  const int nstrip = (w1 + 3) >> 2;
-  const int gsh = group_shift(nstrip);
+  const int h1 = (H + 1) >> 1;
+  const int nitem = W >> 2;                     // 4-column pieces per row
+  const int gsh = group_shift(nitem);
   const int s = tid & ((1 << gsh) - 1);
-  if (s >= nstrip) return;
-  const int c0 = 8 * s;
+  if (s >= nitem) return;
+  const int c0 = 4 * s;
   for (int i = tid >> gsh; i < h1; i += nthreads >> gsh) {
-    float r0[8], r1[8];
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const int cc = c0 + 4 * hf;
-      float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
-      if (cc < W) {
-        load4<T>(src + (2 * i) * W + cc, a);
-        if (2 * i + 1 < H) load4<T>(src + (2 * i + 1) * W + cc, b);
-      }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) { r0[4 * hf + k] = a[k]; r1[4 * hf + k] = b[k]; }
-    }
+    float a[4], b[4] = {0.f, 0.f, 0.f, 0.f};
+    const bool has_b = 2 * i + 1 < H;
+    load4<T>(src + (2 * i) * W + c0, a);
+    if (has_b) load4<T>(src + (2 * i + 1) * W + c0, b);
     float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
-    float* o = d1 + (i + P1) * str1 + 4 * s + P1;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      if (c0 + k < W) {
-        x0[k] = r0[k];
-        if (2 * i + 1 < H) x0[str0 + k] = r1[k];
-      }
+    for (int k = 0; k < 4; ++k) {
+      x0[k] = a[k];
+      if (has_b) x0[str0 + k] = b[k];
     }
+    float* o = d1 + (i + P1) * str1 + 2 * s + P1;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      if (4 * s + t < w1) {
-        const float a = r0[2 * t], b = r0[2 * t + 1], c = r1[2 * t], d = r1[2 * t + 1];
-        const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
+    for (int t = 0; t < 2; ++t) {
+      const float sac = a[2 * t] + b[2 * t], sbd = a[2 * t + 1] + b[2 * t + 1];
+      const float dac = a[2 * t] - b[2 * t], dbd = a[2 * t + 1] - b[2 * t + 1];
+      o[t] = 0.5f * (sac + sbd);
+      o[pl1 + t] = 0.5f * (dac + dbd);
+      o[2 * pl1 + t] = 0.5f * (sac - sbd);
+      o[3 * pl1 + t] = 0.5f * (dac - dbd);
+    }
+  }
+}
+
+// The same work split in two, so that the HBM reads of the next plane are in flight while
+// the current one is computed: plane_fetch issues the loads into registers (NP passes of
+// one 2x4 piece per thread), plane_commit writes level 0 and level 1 into LDS.
+template <typename T, int NP>
+__device__ __forceinline__ void plane_fetch(const T* __restrict__ src, int H, int W, int tid, int nthreads,
+                                            float (&a)[NP][4], float (&b)[NP][4]) {
+  const int h1 = (H + 1) >> 1;
+  const int nitem = W >> 2;
+  const int gsh = group_shift(nitem);
+  const int s = tid & ((1 << gsh) - 1);
+  if (s >= nitem) return;
+  const int c0 = 4 * s;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int i = (tid >> gsh) + p * (nthreads >> gsh);
+    if (i < h1) {
+      // both loads unconditional (no merge with constants, hence no wait right behind the
+      // load); a missing bottom row re-reads the top one and is zeroed in plane_commit
+      const int rb = 2 * i + 1 < H ? 2 * i + 1 : 2 * i;
+      load4<T>(src + (2 * i) * W + c0, a[p]);
+      load4<T>(src + rb * W + c0, b[p]);
+    }
+  }
+}
+
+template <int NP>
+__device__ __forceinline__ void plane_commit(const float (&a)[NP][4], const float (&b)[NP][4], int H, int W,
+                                             float* __restrict__ d0, int str0, int P0,
+                                             float* __restrict__ d1, int str1, int pl1, int P1,
+                                             int tid, int nthreads) {
+  const int h1 = (H + 1) >> 1;
+  const int nitem = W >> 2;
+  const int gsh = group_shift(nitem);
+  const int s = tid & ((1 << gsh) - 1);
+  if (s >= nitem) return;
+  const int c0 = 4 * s;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int i = (tid >> gsh) + p * (nthreads >> gsh);
+    if (i < h1) {
+      const bool has_b = 2 * i + 1 < H;
+      float bb[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) bb[k] = has_b ? b[p][k] : 0.f;
+      float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x0[k] = a[p][k];
+        if (has_b) x0[str0 + k] = bb[k];
+      }
+      float* o = d1 + (i + P1) * str1 + 2 * s + P1;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const float sac = a[p][2 * t] + bb[2 * t], sbd = a[p][2 * t + 1] + bb[2 * t + 1];
+        const float dac = a[p][2 * t] - bb[2 * t], dbd = a[p][2 * t + 1] - bb[2 * t + 1];
         o[t] = 0.5f * (sac + sbd);
         o[pl1 + t] = 0.5f * (dac + dbd);
         o[2 * pl1 + t] = 0.5f * (sac - sbd);
@@ -447,53 +504,77 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 }
 
 // Forward (and, with flipped folded weights and zero fb, input-gradient) kernel.
-// grid.x = B*C planes, block = 256 threads.
+// Persistent: grid.x = min(B*C, resident workgroups), block = 256 threads; a workgroup
+// walks planes blockIdx.x, blockIdx.x + gridDim.x, ...  The zero halos written once stay
+// valid for every plane (only interiors are rewritten).
 template <typename T, int K, int TJ1, int TJC>
 __global__ __launch_bounds__(256) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                          const float* __restrict__ fw,
                                                          const float* __restrict__ fb, Plan2D pl) {
   WT_SHARED_FLOATS(lds);
   constexpr int KK = K * K;
-  const int plane = blockIdx.x;
-  const int c = plane % pl.C;
   const int NF = 1 + 4 * pl.L;
-  wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
-  const size_t plane_off = static_cast<size_t>(plane) * pl.H * pl.W;
+  const size_t plane_elems = static_cast<size_t>(pl.H) * pl.W;
+  const int tid = threadIdx.x;
 
+  WT_TICK_INIT();
   zero_lds(lds, pl.lds_floats);
-  __syncthreads();
-  int l0 = 1;
-  if (pl.vec_ok) {
-    load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
-                      lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, threadIdx.x, blockDim.x);
-    l0 = 2;
-  } else {
-    load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, false);
+  float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
+  if (pl.prefetch) plane_fetch<T, kFetchPasses>(x + blockIdx.x * plane_elems, pl.H, pl.W, tid, blockDim.x, fa, fbuf);
+  WT_LDS_BARRIER();
+  WT_TICK(0);
+  for (int pv = blockIdx.x; pv < pl.nplanes; pv += gridDim.x) {
+    const int plane = WT_UNIFORM(pv);
+    const int c = plane % pl.C;
+    wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
+    const size_t plane_off = static_cast<size_t>(plane) * plane_elems;
+    int l0 = 2;
+    if (pl.prefetch) {
+      plane_commit<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
+                                 lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, tid, blockDim.x);
+    } else if (pl.vec_ok) {
+      load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
+                        lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, tid, blockDim.x);
+    } else {
+      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, false);
+      l0 = 1;
+    }
+    WT_LDS_BARRIER();
+    WT_TICK(1);
+    if (pl.prefetch && plane + static_cast<int>(gridDim.x) < pl.nplanes)
+      plane_fetch<T, kFetchPasses>(x + plane_off + gridDim.x * plane_elems, pl.H, pl.W, tid, blockDim.x, fa, fbuf);
+    for (int lv = l0; lv <= pl.L; ++lv) {
+      const int l = WT_UNIFORM(lv);
+      const float* src = lds + pl.aoff[l - 1];   // sub-band 0 (or the input plane)
+      analysis_level(src, pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
+                     pl.h[l], pl.w[l], tid, blockDim.x);
+      WT_LDS_BARRIER();
+    }
+    WT_TICK(2);
+    for (int lv = pl.L; lv >= 2; --lv) {
+      const int l = WT_UNIFORM(lv);
+      synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK);
+      WT_LDS_BARRIER();
+      WT_TICK(1 + l);
+    }
+    WT_WAIT_VMEM();     // next plane's loads have landed; the stores below are not waited for
+    synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off);
+    WT_LDS_BARRIER();   // the next plane overwrites the buffers read above
+    WT_TICK(7);
   }
-  __syncthreads();
-  for (int lv = l0; lv <= pl.L; ++lv) {
-    const int l = WT_UNIFORM(lv);
-    const float* src = lds + pl.aoff[l - 1];   // sub-band 0 (or the input plane)
-    analysis_level(src, pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
-                   pl.h[l], pl.w[l], threadIdx.x, blockDim.x);
-    __syncthreads();
-  }
-  for (int lv = pl.L; lv >= 2; --lv) {
-    const int l = WT_UNIFORM(lv);
-    synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK);
-    __syncthreads();
-  }
-  synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off);
 }
 
 // ------------------------------------------------------------------ parameter gradients
 // grid = (C, nchunk), block = 512 threads = 8 waves.  Each workgroup walks `bchunk`
-// planes of one channel; wave w accumulates, in registers, the K*K correlation sums of
-// sub-band (w & 3) at every level plus its share of the base-conv sums.  One cross-lane
-// reduction at the end, partial sums to HBM, finished by wgrad_finish_kernel (two-stage,
-// deterministic; the reference uses float atomics, fused_haar_conv.cu:331-341).
+// planes of one channel and keeps K*K correlation sums per filter in registers:
 //   dWt_l[c,s,kh,kw] = sum_{b,i,j} dY_l[s][i,j] * A_l[s][i+kh-R, j+kw-R]
 //   dWt_b[c,kh,kw]   = sum_{b,i,j} G[i,j] * x[i+kh-R, j+kw-R],   sumG[c] = sum G
+// The filters are split over the waves so that no thread carries more than three sets:
+//   waves 0-3 ("A", sub-band/quarter q = wave):   base conv rows of quarter q, level 3, level 5
+//   waves 4-7 ("B", sub-band q = wave - 4):       level 1, level 2, level 4
+// One cross-lane reduction at the end, partial sums to HBM, finished by
+// wgrad_finish_kernel (two-stage and deterministic; the reference accumulates with float
+// atomics, fused_haar_conv.cu:331-341).
 template <int K, int TJ, int VW>
 __device__ __forceinline__ void corr_strip(const float* __restrict__ a, int astr,
                                            const float* __restrict__ gy, float (&acc)[K * K]) {
@@ -514,6 +595,28 @@ __device__ __forceinline__ void corr_strip(const float* __restrict__ a, int astr
   WT_CHUNK_FENCE();
 }
 
+// Correlation sums of one sub-band plane of one level, walked by a single wave.
+// row0/row_step select the rows this wave owns (all rows: 0 / rows-per-pass).
+template <int K, int TJ, int VW>
+__device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr, const float* __restrict__ G,
+                                           int gstr, int h, int w, int lane, int pass_row0, int pass_step,
+                                           float (&acc)[K * K], float gmul, float& gsum) {
+  const int nstrip = (w + TJ - 1) / TJ;
+  const int gsh = group_shift(nstrip);
+  const int strip = lane & ((1 << gsh) - 1);
+  if (strip >= nstrip) return;
+  const int j0 = strip * TJ;
+  const int rpp = kWave >> gsh;          // rows per pass of one wave (>= 1: nstrip <= 64)
+  for (int i = pass_row0 * rpp + (lane >> gsh); i < h; i += pass_step * rpp) {
+    const float* gy = G + i * gstr + j0;
+#pragma unroll
+    for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t], gsum);
+    corr_strip<K, TJ, VW>(A + i * astr + j0, astr, gy, acc);   // A already points R rows/cols up-left
+  }
+}
+
+constexpr int wgrad_sets(int L) { return L >= 4 ? 3 : (L >= 2 ? 2 : 1); }
+
 template <typename T, int K, int L, int TJ>
 __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
                                                          float* __restrict__ partial, Plan2D pl,
@@ -523,26 +626,29 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
   constexpr int R = K / 2;
   constexpr int NF = 1 + 4 * L;
   constexpr int VW = (R >= 1 && TJ % 4 == 0) ? 4 : 1;
+  constexpr int NSET = wgrad_sets(L);
   const int c = blockIdx.x;
   const int chunk = blockIdx.y;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int sb = wave & 3;
-  const int sub_tid = (wave >> 2) * kWave + (tid & (kWave - 1));   // 0..127 within the sub-band group
+  const int wave = WT_UNIFORM(tid >> 6);
+  const int lane = tid & (kWave - 1);
+  const int q = wave & 3;
+  const bool role_a = wave < 4;
   const int P = pl.P;
 
-  float accb[KK];
-  float accl[L][KK];
+  float acc[NSET][KK];
   float gsum = 0.f;
 #pragma unroll
-  for (int t = 0; t < KK; ++t) accb[t] = 0.f;
+  for (int s = 0; s < NSET; ++s)
 #pragma unroll
-  for (int l = 0; l < L; ++l)
-#pragma unroll
-    for (int t = 0; t < KK; ++t) accl[l][t] = 0.f;
+    for (int t = 0; t < KK; ++t) acc[s][t] = 0.f;
 
   zero_lds(lds, pl.lds_floats);
-  __syncthreads();
+  WT_LDS_BARRIER();
+
+  // pointers to the top-left corner of the conv window of element (0,0)
+  auto a_plane = [&](int l, int s) { return lds + pl.aoff[l] + s * pl.apl[l] + (P - R) * pl.astr[l] + (P - R); };
+  auto g_plane = [&](int l, int s) { return lds + pl.goff[l] + s * pl.gpl[l]; };
 
   const int b_end = (chunk + 1) * bchunk < B ? (chunk + 1) * bchunk : B;
   for (int bv = chunk * bchunk; bv < b_end; ++bv) {
@@ -559,90 +665,72 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
       load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, false);
       load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, false);
     }
-    __syncthreads();
+    WT_LDS_BARRIER();
     for (int lv = l0; lv <= L; ++lv) {
       const int l = WT_UNIFORM(lv);
       analysis_level(lds + pl.aoff[l - 1], pl.astr[l - 1], P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], P,
                      pl.h[l], pl.w[l], tid, blockDim.x);
       analysis_level(lds + pl.goff[l - 1], pl.gstr[l - 1], 0, lds + pl.goff[l], pl.gstr[l], pl.gpl[l], 0,
                      pl.h[l], pl.w[l], tid, blockDim.x);
-      __syncthreads();
+      WT_LDS_BARRIER();
     }
-    {  // base conv: all threads share the full-resolution plane
-      const int nstrip = (pl.W + TJ - 1) / TJ;
-      const int gsh = group_shift(nstrip);
-      const int strip = tid & ((1 << gsh) - 1);
-      if (strip < nstrip) {
-        const int j0 = strip * TJ;
-        const float* X = lds + pl.aoff[0] + (j0 - R + P);
-        const float* G = lds + pl.goff[0] + j0;
-        for (int i = tid >> gsh; i < pl.H; i += blockDim.x >> gsh) {
-          const float* gy = G + i * pl.gstr[0];
-#pragma unroll
-          for (int t = 0; t < TJ; ++t) gsum += gy[t];
-          corr_strip<K, TJ, VW>(X + (i - R + P) * pl.astr[0], pl.astr[0], gy, accb);
-        }
+    // Both roles run the same code on different planes (one code path keeps a single
+    // register set for the sums): level index per set, -1 = base conv, 0 = nothing.
+    {
+      const int l = role_a ? 0 : 1;            // set 0, strips of TJ: base conv rows (A) / level 1 (B)
+      corr_level<K, TJ, VW>(a_plane(l, role_a ? 0 : q), pl.astr[l], g_plane(l, role_a ? 0 : q), pl.gstr[l],
+                            pl.h[l], pl.w[l], lane, role_a ? q : 0, role_a ? 4 : 1, acc[0], role_a ? 1.f : 0.f,
+                            gsum);
+    }
+    if constexpr (NSET >= 2) {                 // set 1, single coefficients: level 3 (A) / level 2 (B)
+      const int l = role_a ? 3 : 2;
+      if (l <= L) {
+        float unused = 0.f;
+        corr_level<K, 1, 1>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], pl.h[l], pl.w[l], lane, 0, 1,
+                            acc[1], 0.f, unused);
       }
     }
-    {  // level 1: strips of TJ; the two waves of a sub-band share its rows
-      const int nstrip = (pl.w[1] + TJ - 1) / TJ;
-      const int gsh = group_shift(nstrip);
-      const int strip = sub_tid & ((1 << gsh) - 1);
-      if (strip < nstrip) {
-        const int j0 = strip * TJ;
-        const float* A = lds + pl.aoff[1] + sb * pl.apl[1] + (j0 - R + P);
-        const float* G = lds + pl.goff[1] + sb * pl.gpl[1] + j0;
-        for (int i = sub_tid >> gsh; i < pl.h[1]; i += (2 * kWave) >> gsh)
-          corr_strip<K, TJ, VW>(A + (i - R + P) * pl.astr[1], pl.astr[1], G + i * pl.gstr[1], accl[0]);
+    if constexpr (NSET >= 3) {                 // set 2: level 5 (A) / level 4 (B)
+      const int l = role_a ? 5 : 4;
+      if (l <= L) {
+        float unused = 0.f;
+        corr_level<K, 1, 1>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], pl.h[l], pl.w[l], lane, 0, 1,
+                            acc[2], 0.f, unused);
       }
     }
-#pragma unroll
-    for (int l = 2; l <= L; ++l) {   // coarse levels: one coefficient per item keeps the lanes busy
-      const int gsh = group_shift(pl.w[l]);
-      const int j0 = sub_tid & ((1 << gsh) - 1);
-      if (j0 < pl.w[l]) {
-        const float* A = lds + pl.aoff[l] + sb * pl.apl[l] + (j0 - R + P);
-        const float* G = lds + pl.goff[l] + sb * pl.gpl[l] + j0;
-        for (int i = sub_tid >> gsh; i < pl.h[l]; i += (2 * kWave) >> gsh)
-          corr_strip<K, 1, 1>(A + (i - R + P) * pl.astr[l], pl.astr[l], G + i * pl.gstr[l], accl[l - 1]);
-      }
-    }
-    __syncthreads();
+    WT_LDS_BARRIER();
   }
 
   // cross-lane reduction, then cross-wave through LDS (pyramid buffers are dead now)
-  constexpr int NRED = KK * (L + 1) + 1;
+  constexpr int NRED = NSET * KK + 1;
   float* red = lds;   // [8 waves][NRED]
-  const int lane = tid & (kWave - 1);
 #pragma unroll
-  for (int t = 0; t < KK; ++t) {
-    const float v = wave_sum(accb[t]);
-    if (lane == 0) red[wave * NRED + t] = v;
-  }
-#pragma unroll
-  for (int l = 0; l < L; ++l)
+  for (int s = 0; s < NSET; ++s)
 #pragma unroll
     for (int t = 0; t < KK; ++t) {
-      const float v = wave_sum(accl[l][t]);
-      if (lane == 0) red[wave * NRED + KK * (l + 1) + t] = v;
+      const float v = wave_sum(acc[s][t]);
+      if (lane == 0) red[wave * NRED + s * KK + t] = v;
     }
   {
     const float v = wave_sum(gsum);
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
-  __syncthreads();
+  WT_LDS_BARRIER();
   float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * (NF * KK + 1);
   for (int o = tid; o < NF * KK + 1; o += blockDim.x) {
     float v = 0.f;
     if (o == NF * KK) {
-      for (int wv = 0; wv < 8; ++wv) v += red[wv * NRED + NRED - 1];
+      for (int wv = 0; wv < 4; ++wv) v += red[wv * NRED + NRED - 1];
     } else {
       const int f = o / KK, t = o - f * KK;
       if (f == 0) {
-        for (int wv = 0; wv < 8; ++wv) v += red[wv * NRED + t];
+        for (int wv = 0; wv < 4; ++wv) v += red[wv * NRED + t];
       } else {
-        const int l = (f - 1) >> 2, s = (f - 1) & 3;
-        v = red[s * NRED + KK * (l + 1) + t] + red[(s + 4) * NRED + KK * (l + 1) + t];
+        const int l = 1 + ((f - 1) >> 2), s = (f - 1) & 3;
+        // level -> (role, set): 1 -> B0, 2 -> B1, 3 -> A1, 4 -> B2, 5 -> A2
+        const bool in_a = (l == 3) || (l == 5);
+        const int set = l == 1 ? 0 : (l <= 3 ? 1 : 2);
+        v = red[(in_a ? s : 4 + s) * NRED + set * KK + t];
       }
     }
     dst[o] = v;

@@ -18,10 +18,11 @@ constexpr int kTJW = 4;     // weight-gradient correlation strips
 
 // Fills the LDS layout of one plane.  with_grad_pyramid adds the padded pyramid of
 // grad_out used by the weight-gradient kernel (and drops the Z buffers it does not need).
-inline Plan2D make_plan2d(int C, int H, int W, int K, int L, bool with_grad_pyramid,
+inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
                           size_t elem_size, const void* p0, const void* p1, const void* p2) {
   Plan2D pl = {};
   pl.C = C; pl.H = H; pl.W = W; pl.L = L;
+  pl.nplanes = B * C;
   const int R = K / 2;
   pl.P = R > 1 ? R : 1;
   pl.h[0] = H; pl.w[0] = W;
@@ -51,6 +52,13 @@ inline Plan2D make_plan2d(int C, int H, int W, int K, int L, bool with_grad_pyra
   const uintptr_t mask = 4 * elem_size - 1;       // 4-element vectors: 16 B (fp32) / 8 B (bf16)
   auto aligned = [mask](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
   pl.vec_ok = (W % 4 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
+  if (pl.vec_ok) {
+    // 2x4 pieces per row-pair, walked by groups of the next power of two of W/4 lanes
+    int gs = 1;
+    while (gs < W / 4) gs *= 2;
+    const int rows_per_pass = nthreads / gs;
+    pl.prefetch = rows_per_pass >= 1 && (pl.h[1] + rows_per_pass - 1) / rows_per_pass <= kFetchPasses;
+  }
   return pl;
 }
 
@@ -114,6 +122,15 @@ inline void wgrad_chunks1d(int B, int C, int ntiles, int* per_chunk, int* nchunk
   if (pc < 1) pc = 1;
   *per_chunk = pc;
   *nchunk = (total + pc - 1) / pc;
+}
+
+// Workgroups of a persistent kernel: as many as can be resident at once.
+inline int resident_workgroups(int ncu, size_t lds_bytes, int waves_per_wg, int max_waves_per_simd) {
+  const int by_lds = lds_bytes ? static_cast<int>(kLdsLimitBytes / lds_bytes) : 8;
+  const int by_waves = (4 * max_waves_per_simd) / waves_per_wg;
+  int per_cu = by_lds < by_waves ? by_lds : by_waves;
+  if (per_cu < 1) per_cu = 1;
+  return ncu * per_cu;
 }
 
 }  // namespace wt
