@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary dtype and per-kernel timing")
     ap.add_argument("--cpu-batch", type=int, default=16)
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="only run a plain device copy of one activation tensor (calibrates rocprof's "
+                         "FETCH_SIZE/WRITE_SIZE against a kernel of known traffic) and exit")
     return ap.parse_args()
 
 
@@ -210,6 +213,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     C, H, W, K, L, B = WORKLOADS[args.workload]
+
+    if args.probe_copy:
+        dt = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+        src = torch.randn(B, C, H, W, device=dev).to(dt)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy", "bytes_read": src.numel() * src.element_size(),
+                          "bytes_written": src.numel() * src.element_size(), "launches": args.warmup + args.steps}))
+        return
 
     main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup,
                            per_kernel=not args.no_extra)
