@@ -161,6 +161,44 @@ def bench_layer(torch, dev, dtype_name, workload, steps, warmup, per_kernel=True
     return res
 
 
+def bench_1d(torch, dev, steps, warmup):
+    """BASELINE config 4: WTConv1d(64,64,5,wt_levels=4), fp32, fwd+bwd, x[64,64,4096]."""
+    from wtconv.wtconv1d import WTConv1d
+    B, C, N, K, L = 64, 64, 4096, 5, 4
+    P = B * C * N
+    torch.manual_seed(0)
+    mod = WTConv1d(C, C, K, wt_levels=L).to(dev)
+    nsets = max(3, int(600e6 // (3 * P * 4)) + 1)
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    sets = [(torch.randn(B, C, N, generator=gen).to(dev).requires_grad_(True), torch.randn(B, C, N, generator=gen).to(dev))
+            for _ in range(nsets)]
+
+    def step(i):
+        x, g = sets[i]
+        x.grad = None
+        for p in mod.parameters():
+            p.grad = None
+        mod(x).backward(g)
+
+    wall_ms, med_ms, _, _ = time_steps(torch, step, nsets, steps, warmup)
+    return {"workload": f"WTConv1d({C},{C},kernel_size={K},wt_levels={L}) fwd+bwd on x[{B},{C},{N}] fp32",
+            "ms_per_step": wall_ms, "sequences_per_s": B / (wall_ms * 1e-3),
+            "step_GBps": 5 * P * 4 / (wall_ms * 1e-3) / 1e9,
+            "step_frac_hbm": 5 * P * 4 / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+
+def bench_model(torch, dev, steps, warmup, batch=256):
+    """BASELINE config 5: WTConvNeXt-T, random init (seed 0), bf16 inference on [batch,3,224,224]."""
+    import wtconvnext
+    torch.manual_seed(0)
+    model = wtconvnext.wtconvnext_tiny().to(dev).bfloat16().eval()
+    x = torch.randn(batch, 3, 224, 224, device=dev).bfloat16()
+    with torch.no_grad():
+        wall_ms, med_ms, _, _ = time_steps(torch, lambda i: model(x), 1, steps, warmup)
+    return {"workload": f"WTConvNeXt-T bf16 inference forward, batch {batch}, 3x224x224, WTConv layers on the HIP kernels",
+            "ms_per_step": wall_ms, "images_per_s": batch / (wall_ms * 1e-3)}
+
+
 def cpu_baseline(torch, workload, cpu_batch):
     """The CPU oracle (torch.nn.functional restatement of the reference layer) forward +
     backward in fp32 on all host cores, on `cpu_batch` images of the same shape."""
@@ -255,6 +293,14 @@ def main():
         other = "bf16" if args.dtype == "fp32" else "fp32"
         o = bench_layer(torch, dev, other, args.workload, args.steps, args.warmup, per_kernel=False)
         line["other_dtype"] = {k: o[k] for k in ("dtype", "ms_per_step", "images_per_s", "step_GBps", "step_frac_hbm")}
+        if args.workload == "stage1":
+            sweep = {}
+            for wl in ("stage2", "stage3", "stage4"):
+                o = bench_layer(torch, dev, "bf16", wl, max(10, args.steps // 2), max(3, args.warmup // 2), per_kernel=False)
+                sweep[wl] = {k: o[k] for k in ("dtype", "ms_per_step", "images_per_s", "step_GBps", "step_frac_hbm")}
+            line["stage_sweep_bf16"] = sweep
+            line["wtconv1d"] = bench_1d(torch, dev, max(10, args.steps // 2), max(3, args.warmup // 2))
+            line["wtconvnext_t"] = bench_model(torch, dev, 5, 2)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, args.workload, args.cpu_batch)
     print(json.dumps(line))

@@ -206,3 +206,57 @@ def test_config2_full_size_param_grads_vs_oracle(hip_device):
         e_hip = (gg[n].double() - want).abs().max().item()
         e_cpu = (wg32[n].double() - want).abs().max().item()
         print(f"\n{n}: max|hip-fp64| = {e_hip:.3e}, max|cpu_fp32-fp64| = {e_cpu:.3e}, max|want| = {want.abs().max():.1f}")
+
+
+# ------------------------------------------------------------------ caller harness
+def test_wtconvnext_harness_hip_vs_oracle_conv_class(hip_device):
+    """WTConvNeXt-T (reduced depth) with the HIP WTConv2d against the same host model with the
+    oracle conv class (same seed, same state dict): logits and input gradient, fp32."""
+    import wtconvnext
+    from oracle import wtconv_ref as R
+    torch.manual_seed(0)
+    ref = wtconvnext.wtconvnext_tiny(depths=(1, 1, 2, 1), num_classes=16, wtconv_class=R.RefWTConv2d,
+                                     ls_init_value=1.0)
+    U_gen = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        for n, p in ref.named_parameters():
+            if "wavelet_scale" in n or "base_scale" in n:
+                p.copy_(torch.rand(p.shape, generator=U_gen) + 0.5)
+    hip = wtconvnext.wtconvnext_tiny(depths=(1, 1, 2, 1), num_classes=16, ls_init_value=1.0)
+    hip.load_state_dict(ref.state_dict(), strict=True)
+    hip = hip.to(hip_device)
+    x = torch.randn(2, 3, 224, 224)
+    xr = x.clone().requires_grad_(True)
+    yr = ref(xr)
+    yr.sum().backward()
+    xh = x.to(hip_device).requires_grad_(True)
+    yh = hip(xh)
+    yh.sum().backward()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(yh.detach().cpu(), yr.detach(), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(xh.grad.cpu(), xr.grad, rtol=1e-3, atol=1e-5)
+    g_ref = dict(ref.named_parameters())
+    for n, p in hip.named_parameters():
+        if "conv_dw" in n and p.grad is not None:
+            torch.testing.assert_close(p.grad.cpu(), g_ref[n].grad, rtol=1e-3, atol=1e-4, msg=lambda m, n=n: f"{n}: {m}")
+
+
+def test_wtconvnext_tiny_bf16_inference_runs(hip_device):
+    """The BASELINE config-5 model at a small batch: bf16 inference forward on the HIP layer,
+    compared with the same bf16 model using the oracle conv class on the GPU (cuDNN-free
+    torch ops), loose tolerance (bf16 end to end)."""
+    import wtconvnext
+    from oracle import wtconv_ref as R
+    torch.manual_seed(0)
+    ref = wtconvnext.wtconvnext_tiny(wtconv_class=R.RefWTConv2d, ls_init_value=1.0)
+    hip = wtconvnext.wtconvnext_tiny(ls_init_value=1.0)
+    hip.load_state_dict(ref.state_dict(), strict=True)
+    hip = hip.to(hip_device).bfloat16().eval()
+    x = torch.randn(4, 3, 224, 224)
+    with torch.no_grad():
+        yr = ref.eval()(x)                     # fp32 CPU oracle model
+        yh = hip(x.to(hip_device).bfloat16()).float().cpu()
+    rms = yr.pow(2).mean().sqrt().item()
+    err = (yh - yr).pow(2).mean().sqrt().item()
+    print(f"\nbf16 HIP model vs fp32 oracle model: rms err {err:.3e}, rms {rms:.3e}")
+    assert err <= 5e-2 * rms
