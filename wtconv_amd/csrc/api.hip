@@ -63,6 +63,24 @@ static int compute_units() {
 #endif
 }
 
+// Workgroups of `kernel` that fit on one CU at once (registers, LDS, wave slots): the grid
+// of a persistent kernel must not exceed CUs x this, or the surplus runs as a second round.
+template <typename F>
+static int resident_per_cu(F kernel, int block, size_t lds_bytes) {
+#ifdef WT_EMULATE
+  (void)kernel; (void)block; (void)lds_bytes;
+  return 1;
+#else
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kernel), block, lds_bytes) !=
+          hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = resident_workgroups(1, lds_bytes, block / 64, 8);
+  }
+  return n;
+#endif
+}
+
 static ParamTable to_table(const wtconv_params* p, int L) {
   ParamTable t = {};
   t.base_weight = p->base_weight;
@@ -102,27 +120,40 @@ static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float
   return check_launch("fold_params_kernel");
 }
 
-// ---- 2-D dispatch over (dtype, K) ---------------------------------------------------
-template <typename T, int K>
-static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl, int B,
+// ---- 2-D dispatch over (dtype, K, level-1 strip width) -------------------------------
+template <typename T, int K, int TJ1>
+static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
                        hipStream_t stream) {
-  auto kern = wt2d_plane_kernel<T, K, kTJ1, kTJC>;
+  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
-  int nwg = resident_workgroups(compute_units(), lds, 4, 8);
-  if (nwg > B * pl.C) nwg = B * pl.C;
+  const int sg = 1 << pl.sg_shift;
+  const int slots = 256 / sg;
+  const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
+  int nwg = compute_units() * resident_per_cu(kern, 256, lds);
+  if (nwg > nunits) nwg = nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
 }
 
+template <typename T, int K>
+static int run_plane2d_tj(int tj1, const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
+                          hipStream_t stream) {
+  switch (tj1) {
+    case 1: return run_plane2d<T, K, 1>(x, out, fw, fb, pl, stream);
+    case 2: return run_plane2d<T, K, 2>(x, out, fw, fb, pl, stream);
+    default: return run_plane2d<T, K, 4>(x, out, fw, fb, pl, stream);
+  }
+}
+
 template <typename T>
-static int run_plane2d_k(int K, const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
-                         int B, hipStream_t stream) {
+static int run_plane2d_k(int K, int tj1, const void* x, void* out, const float* fw, const float* fb,
+                         const Plan2D& pl, hipStream_t stream) {
   switch (K) {
-    case 1: return run_plane2d<T, 1>(x, out, fw, fb, pl, B, stream);
-    case 3: return run_plane2d<T, 3>(x, out, fw, fb, pl, B, stream);
-    case 5: return run_plane2d<T, 5>(x, out, fw, fb, pl, B, stream);
-    case 7: return run_plane2d<T, 7>(x, out, fw, fb, pl, B, stream);
+    case 1: return run_plane2d_tj<T, 1>(tj1, x, out, fw, fb, pl, stream);
+    case 3: return run_plane2d_tj<T, 3>(tj1, x, out, fw, fb, pl, stream);
+    case 5: return run_plane2d_tj<T, 5>(tj1, x, out, fw, fb, pl, stream);
+    case 7: return run_plane2d_tj<T, 7>(tj1, x, out, fw, fb, pl, stream);
   }
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
@@ -172,7 +203,12 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  const Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
+  Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
+  int tj1 = 4, sg_shift = 8;
+  choose_plane_shape(pl.h[1], pl.w[1], &tj1, &sg_shift);
+  // keep the slots of a workgroup within LDS: fewer, larger plane groups if needed
+  while (sg_shift < 8 && static_cast<size_t>(pl.plane_lds_floats) * 4 * (256 >> sg_shift) > kLdsLimitBytes / 2) ++sg_shift;
+  finish_plane_plan(&pl, sg_shift);
   if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
     return fail(WTCONV_E_UNSUPPORTED,
                 "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
@@ -184,8 +220,8 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
-  return dtype == WTCONV_F32 ? run_plane2d_k<float>(K, x, out, fw, fb, pl, B, stream)
-                             : run_plane2d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
+  return dtype == WTCONV_F32 ? run_plane2d_k<float>(K, tj1, x, out, fw, fb, pl, stream)
+                             : run_plane2d_k<bf16_t>(K, tj1, x, out, fw, fb, pl, stream);
 }
 
 // ---- 1-D dispatch -------------------------------------------------------------------

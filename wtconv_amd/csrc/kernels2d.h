@@ -41,6 +41,10 @@ struct Plan2D {
   int prefetch;                // vec_ok and a plane is at most kFetchPasses pieces per thread:
                                //   the next plane is fetched into registers during compute
   int nplanes;                 // B * C
+  int B;
+  int sg_shift;                // log2 of the threads that share one plane (4..8)
+  int plane_lds_floats;        // LDS of one plane slot; lds_floats = slots * this
+  int groups_per_channel;      // sg < 64: a wave holds 64/sg planes of one channel; number of such groups per channel
 };
 
 // ------------------------------------------------------------------ parameter folding
@@ -78,37 +82,16 @@ __global__ void fold_params_kernel(ParamTable p, int pdtype, float* __restrict__
 // element (r, col) sits at dst[(r + P) * str + col + P].
 template <typename T>
 __device__ __forceinline__ void load_plane(const T* __restrict__ src, float* __restrict__ dst,
-                                           int H, int W, int str, int P, bool vec) {
-  const int n = H * W;
-  if (vec) {
-    constexpr int EV = 16 / sizeof(T);
-    const int nv = n / EV;
-    const uint4* __restrict__ s4 = reinterpret_cast<const uint4*>(src);
-    for (int v = threadIdx.x; v < nv; v += blockDim.x) {
-      const uint4 q = s4[v];
-      float vals[EV];
-      if constexpr (sizeof(T) == 4) {
-        vals[0] = __uint_as_float(q.x); vals[1] = __uint_as_float(q.y);
-        vals[2] = __uint_as_float(q.z); vals[3] = __uint_as_float(q.w);
-      } else {
-        const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          vals[2 * k] = __uint_as_float(qq[k] << 16);
-          vals[2 * k + 1] = __uint_as_float(qq[k] & 0xffff0000u);
-        }
-      }
-      const int e = v * EV;
-      int r = e / W;
-      int col = e - r * W;
-#pragma unroll
-      for (int k = 0; k < EV; ++k) {
-        dst[(r + P) * str + col + P] = vals[k];
-        if (++col == W) { col = 0; ++r; }
-      }
-    }
+                                           int H, int W, int str, int P, int tid, int nthreads) {
+  const int gsh = W <= 1 ? 0 : 32 - __clz(W - 1);
+  const int rpp = nthreads >> gsh;
+  if (rpp >= 1) {                      // lane groups of 2^gsh >= W lanes walk whole rows
+    const int col = tid & ((1 << gsh) - 1);
+    if (col >= W || (tid >> gsh) >= rpp) return;
+    for (int r = tid >> gsh; r < H; r += rpp) dst[(r + P) * str + col + P] = to_f32<T>(src[r * W + col]);
   } else {
-    for (int e = threadIdx.x; e < n; e += blockDim.x) {
+    const int n = H * W;
+    for (int e = tid; e < n; e += nthreads) {
       const int r = e / W, col = e - r * W;
       dst[(r + P) * str + col + P] = to_f32<T>(src[e]);
     }
@@ -246,9 +229,24 @@ __device__ __forceinline__ void analysis_level(const float* __restrict__ src, in
                                                float* __restrict__ dst, int dstr, int dpl, int dP,
                                                int hl, int wl, int tid, int nthreads) {
   const int gsh = group_shift(wl);
+  const int rpp = nthreads >> gsh;
+  if (rpp == 0) {   // a row is wider than the lane group: plain strided walk
+    for (int it = tid; it < hl * wl; it += nthreads) {
+      const int i = it / wl, j = it - i * wl;
+      const float* s0 = src + (2 * i + sP) * sstr + 2 * j + sP;
+      const float a = s0[0], b = s0[1], c = s0[sstr], d = s0[sstr + 1];
+      const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
+      float* o = dst + (i + dP) * dstr + j + dP;
+      o[0] = 0.5f * (sac + sbd);
+      o[dpl] = 0.5f * (dac + dbd);
+      o[2 * dpl] = 0.5f * (sac - sbd);
+      o[3 * dpl] = 0.5f * (dac - dbd);
+    }
+    return;
+  }
   const int j = tid & ((1 << gsh) - 1);
   if (j >= wl) return;
-  for (int i = tid >> gsh; i < hl; i += nthreads >> gsh) {
+  for (int i = tid >> gsh; i < hl; i += rpp) {
     const float* s0 = src + (2 * i + sP) * sstr + 2 * j + sP;
     const float a = s0[0], b = s0[1], c = s0[sstr], d = s0[sstr + 1];
     const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
@@ -360,13 +358,13 @@ __device__ __forceinline__ void ihaar4(float ll, float lh, float hl, float hh,
 // inverse Haar, cropped store into Z_l.
 template <int K, int TJ>
 __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2D& pl, int l,
-                                            wt_uniform_ptr wl_f) {
+                                            wt_uniform_ptr wl_f, int ltid, int nth) {
   constexpr int R = K / 2;
   constexpr int VW = (R >= 1) ? TJ : 1;   // window starts at column j0 when the halo equals R
   const int hl = pl.h[l], wl = pl.w[l];
   const int nstrip = (wl + TJ - 1) / TJ;
   const int gsh = group_shift(nstrip);
-  const int strip = threadIdx.x & ((1 << gsh) - 1);
+  const int strip = ltid & ((1 << gsh) - 1);
   if (strip >= nstrip) return;
   const int j0 = strip * TJ;
   const int astr = pl.astr[l], apl = pl.apl[l], P = pl.P;
@@ -377,7 +375,9 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
   float* Zout = lds + pl.zoff[l];
   const int zout_str = pl.zstr[l];
   const int ho = pl.h[l - 1], wo = pl.w[l - 1];
-  for (int i = threadIdx.x >> gsh; i < hl; i += blockDim.x >> gsh) {
+  const int rpp = (nth >> gsh) > 0 ? (nth >> gsh) : 1;
+  if ((ltid >> gsh) >= rpp) return;            // more strips than lanes: not used (nth >= 16 >= strips)
+  for (int i = ltid >> gsh; i < hl; i += rpp) {
     float o0[2 * TJ], o1[2 * TJ];
 #pragma unroll
     for (int t = 0; t < 2 * TJ; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
@@ -395,11 +395,16 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
   }
 }
 
-// Store up to N consecutive outputs (N multiple of 4, destination aligned to 4 elements
-// when vec4 is set); `nvalid` of them lie inside the row.
+// Store up to N consecutive outputs (4-element vectors when N is a multiple of 4, the
+// destination is aligned to 4 elements and vec4 is set); `nvalid` of them lie inside the row.
 template <typename T, int N>
 __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[N], int nvalid, bool vec4) {
-  static_assert(N % 4 == 0, "row pieces are multiples of 4 elements");
+  if constexpr (N % 4 != 0) {
+#pragma unroll
+    for (int e = 0; e < N; ++e)
+      if (e < nvalid) dst[e] = from_f32<T>(v[e]);
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < N / 4; ++k) {
     if (vec4 && 4 * k + 4 <= nvalid) {
@@ -426,7 +431,7 @@ __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[
 template <typename T, int K, int TJ>
 __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2D& pl,
                                             wt_uniform_ptr wb_f, wt_uniform_ptr w1_f, float bias,
-                                            T* __restrict__ out_plane) {
+                                            T* __restrict__ out_plane, int ltid, int nth) {
   constexpr int R = K / 2;
   constexpr int NO = 2 * TJ;
   constexpr int VW = (R >= 1) ? TJ : 1;
@@ -434,7 +439,7 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
   const int hl = pl.h[1], wl = pl.w[1];
   const int nstrip = (wl + TJ - 1) / TJ;
   const int gsh = group_shift(nstrip);
-  const int strip = threadIdx.x & ((1 << gsh) - 1);
+  const int strip = ltid & ((1 << gsh) - 1);
   if (strip >= nstrip) return;
   const int j0 = strip * TJ;
   const int astr = pl.astr[1], apl = pl.apl[1], P = pl.P;
@@ -445,7 +450,9 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
   const float* Zin = lds + pl.zoff[2];
   const int zin_str = pl.zstr[2];
   const int H = pl.H, W = pl.W;
-  for (int i = threadIdx.x >> gsh; i < hl; i += blockDim.x >> gsh) {
+  const int rpp = (nth >> gsh) > 0 ? (nth >> gsh) : 1;
+  if ((ltid >> gsh) >= rpp) return;
+  for (int i = ltid >> gsh; i < hl; i += rpp) {
     float o0[NO], o1[NO];
 #pragma unroll
     for (int t = 0; t < NO; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
@@ -504,61 +511,99 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 }
 
 // Forward (and, with flipped folded weights and zero fb, input-gradient) kernel.
-// Persistent: grid.x = min(B*C, resident workgroups), block = 256 threads; a workgroup
-// walks planes blockIdx.x, blockIdx.x + gridDim.x, ...  The zero halos written once stay
-// valid for every plane (only interiors are rewritten).
+// Persistent: grid.x = min(work units, resident workgroups), block = 256 threads.
+// 2^sg_shift threads share a plane, so a workgroup holds 256 >> sg_shift planes, each in its
+// own LDS slot (small planes: up to 16 per workgroup).  When a plane takes less than a wave,
+// the planes of one wave are the same channel of consecutive batch items, so the folded
+// weights stay wave-uniform (SGPRs).  The zero halos written once stay valid for every plane
+// (only interiors are rewritten).
 template <typename T, int K, int TJ1, int TJC>
-__global__ __launch_bounds__(256) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
+__global__ __launch_bounds__(256, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                          const float* __restrict__ fw,
                                                          const float* __restrict__ fb, Plan2D pl) {
-  WT_SHARED_FLOATS(lds);
+  WT_SHARED_FLOATS(lds_all);
   constexpr int KK = K * K;
   const int NF = 1 + 4 * pl.L;
   const size_t plane_elems = static_cast<size_t>(pl.H) * pl.W;
   const int tid = threadIdx.x;
+  const int sg = 1 << pl.sg_shift;
+  const int ltid = tid & (sg - 1);
+  const int slot = tid >> pl.sg_shift;
+  const int slots = blockDim.x >> pl.sg_shift;
+  float* lds = lds_all + slot * pl.plane_lds_floats;
+  const int wave = tid >> 6;
+  const int ppw = sg < kWave ? kWave >> pl.sg_shift : 1;      // planes per wave
+  const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
+
+  // plane of this thread in work unit u (-1: none) and its (wave-uniform) channel
+  auto locate = [&](int u, int& plane, int& c) {
+    if (sg < kWave) {
+      const int gidx = u * 4 + wave;
+      c = gidx / pl.groups_per_channel;
+      const int b = (gidx - c * pl.groups_per_channel) * ppw + ((tid & (kWave - 1)) >> pl.sg_shift);
+      plane = (c < pl.C && b < pl.B) ? b * pl.C + c : -1;
+      if (c >= pl.C) c = pl.C - 1;
+    } else {
+      plane = u * slots + slot;
+      if (plane >= pl.nplanes) plane = -1;
+      c = plane >= 0 ? plane % pl.C : 0;
+    }
+  };
 
   WT_TICK_INIT();
-  zero_lds(lds, pl.lds_floats);
+  zero_lds(lds_all, pl.lds_floats);
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
-  if (pl.prefetch) plane_fetch<T, kFetchPasses>(x + blockIdx.x * plane_elems, pl.H, pl.W, tid, blockDim.x, fa, fbuf);
+  {
+    int p0, c0;
+    locate(blockIdx.x, p0, c0);
+    if (pl.prefetch && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
+  }
   WT_LDS_BARRIER();
   WT_TICK(0);
-  for (int pv = blockIdx.x; pv < pl.nplanes; pv += gridDim.x) {
-    const int plane = WT_UNIFORM(pv);
-    const int c = plane % pl.C;
+  for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
+    const int u = WT_UNIFORM(uv);
+    int plane, cv;
+    locate(u, plane, cv);
+    const int c = WT_UNIFORM(cv);
+    const bool live = plane >= 0;
     wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
-    const size_t plane_off = static_cast<size_t>(plane) * plane_elems;
+    const size_t plane_off = static_cast<size_t>(live ? plane : 0) * plane_elems;
     int l0 = 2;
     if (pl.prefetch) {
-      plane_commit<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
-                                 lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, tid, blockDim.x);
+      if (live)
+        plane_commit<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
+                                   lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, ltid, sg);
     } else if (pl.vec_ok) {
-      load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
-                        lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, tid, blockDim.x);
+      if (live)
+        load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
+                          lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, ltid, sg);
     } else {
-      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, false);
+      if (live) load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, ltid, sg);
       l0 = 1;
     }
     WT_LDS_BARRIER();
     WT_TICK(1);
-    if (pl.prefetch && plane + static_cast<int>(gridDim.x) < pl.nplanes)
-      plane_fetch<T, kFetchPasses>(x + plane_off + gridDim.x * plane_elems, pl.H, pl.W, tid, blockDim.x, fa, fbuf);
+    if (pl.prefetch && u + static_cast<int>(gridDim.x) < nunits) {
+      int pn, cn;
+      locate(u + gridDim.x, pn, cn);
+      if (pn >= 0) plane_fetch<T, kFetchPasses>(x + pn * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
+    }
     for (int lv = l0; lv <= pl.L; ++lv) {
       const int l = WT_UNIFORM(lv);
-      const float* src = lds + pl.aoff[l - 1];   // sub-band 0 (or the input plane)
-      analysis_level(src, pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
-                     pl.h[l], pl.w[l], tid, blockDim.x);
+      if (live)
+        analysis_level(lds + pl.aoff[l - 1], pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
+                       pl.h[l], pl.w[l], ltid, sg);
       WT_LDS_BARRIER();
     }
     WT_TICK(2);
     for (int lv = pl.L; lv >= 2; --lv) {
       const int l = WT_UNIFORM(lv);
-      synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK);
+      if (live) synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK, ltid, sg);
       WT_LDS_BARRIER();
       WT_TICK(1 + l);
     }
     WT_WAIT_VMEM();     // next plane's loads have landed; the stores below are not waited for
-    synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off);
+    if (live) synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off, ltid, sg);
     WT_LDS_BARRIER();   // the next plane overwrites the buffers read above
     WT_TICK(7);
   }
@@ -662,8 +707,8 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
                         lds + pl.goff[1], pl.gstr[1], pl.gpl[1], 0, tid, blockDim.x);
       l0 = 2;
     } else {
-      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, false);
-      load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, false);
+      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, tid, blockDim.x);
+      load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, tid, blockDim.x);
     }
     WT_LDS_BARRIER();
     for (int lv = l0; lv <= L; ++lv) {

@@ -12,54 +12,90 @@ namespace wt {
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Strip widths of the 2-D kernels (outputs per work item along a row).
-constexpr int kTJ1 = 4;     // level 1 (2 x 2*TJ1 output pixels per item)
-constexpr int kTJC = 2;     // coarser levels
+constexpr int kTJC = 2;     // coarser levels of the plane kernel
 constexpr int kTJW = 4;     // weight-gradient correlation strips
 
-// Fills the LDS layout of one plane.  with_grad_pyramid adds the padded pyramid of
-// grad_out used by the weight-gradient kernel (and drops the Z buffers it does not need).
+inline int pow2_ceil(int v) { int p = 1; while (p < v) p *= 2; return p; }
+inline int log2_int(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
+
+// Level-1 strip width and threads per plane of the plane kernel: the pair that keeps most
+// lanes busy in the level-1 phase (ties: the wider strip, which reads less LDS per FMA).
+inline void choose_plane_shape(int h1, int w1, int* tj1, int* sg_shift) {
+  double best = -1.0;
+  for (int tj = 4; tj >= 1; tj /= 2) {
+    const int gs = pow2_ceil((w1 + tj - 1) / tj);
+    int sg = pow2_ceil(gs * h1);
+    if (sg < 16) sg = 16;
+    if (sg > 256) sg = 256;
+    const int rpp = sg / gs > 0 ? sg / gs : 1;
+    const int passes = (h1 + rpp - 1) / rpp;
+    const double eff = static_cast<double>(h1) * w1 / (static_cast<double>(sg) * passes * tj);
+    if (eff > best + 1e-9) { best = eff; *tj1 = tj; *sg_shift = log2_int(sg); }
+  }
+}
+
+// Fills the LDS layout of one plane.  Planes are stacked in one column: x, then the four
+// sub-band planes of level 1, level 2, ...; consecutive planes are separated by one gap of
+// P zero rows that serves as bottom halo of the upper and top halo of the lower plane.
+// with_grad_pyramid adds the padded pyramid of grad_out used by the weight-gradient kernel
+// (and drops the Z buffers it does not need).
 inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
                           size_t elem_size, const void* p0, const void* p1, const void* p2) {
   Plan2D pl = {};
-  pl.C = C; pl.H = H; pl.W = W; pl.L = L;
+  pl.B = B; pl.C = C; pl.H = H; pl.W = W; pl.L = L;
   pl.nplanes = B * C;
   const int R = K / 2;
   pl.P = R > 1 ? R : 1;
   pl.h[0] = H; pl.w[0] = W;
   for (int l = 1; l <= L; ++l) { pl.h[l] = (pl.h[l - 1] + 1) / 2; pl.w[l] = (pl.w[l - 1] + 1) / 2; }
-  int off = 0;
+  // element (r, col) of sub-band s of level l sits at aoff[l] + s*apl[l] + (r+P)*astr[l] + col + P
+  int off = 0;            // start of the zero gap above the next plane
   for (int l = 0; l <= L; ++l) {
     pl.astr[l] = round_up(pl.w[l] + 2 * pl.P, 4);
-    pl.apl[l] = round_up(pl.astr[l] * (pl.h[l] + 2 * pl.P), 4);
+    pl.apl[l] = (pl.h[l] + pl.P) * pl.astr[l];
+    if (l > 0) off += pl.P * (pl.astr[l - 1] - pl.astr[l]);   // the gap keeps the wider stride of the level above
     pl.aoff[l] = off;
     off += pl.apl[l] * (l == 0 ? 1 : 4);
   }
+  off += pl.P * pl.astr[L];                                   // bottom halo of the last plane
   if (!with_grad_pyramid) {
     for (int l = 2; l <= L; ++l) {
-      pl.zstr[l] = round_up(pl.w[l - 1], 4);
+      pl.zstr[l] = pl.w[l - 1];
       pl.zoff[l] = off;
-      off += pl.zstr[l] * pl.h[l - 1];
+      off += round_up(pl.zstr[l] * pl.h[l - 1], 4);
     }
   } else {
     for (int l = 0; l <= L; ++l) {
       pl.gstr[l] = round_up(pl.w[l] + 1, 4);
-      pl.gpl[l] = round_up(pl.gstr[l] * (pl.h[l] + 1), 4);
+      pl.gpl[l] = pl.gstr[l] * (pl.h[l] + 1);
       pl.goff[l] = off;
       off += pl.gpl[l] * (l == 0 ? 1 : 4);
     }
   }
-  pl.lds_floats = round_up(off + kLdsSlackFloats, 4);
+  pl.plane_lds_floats = round_up(off + kLdsSlackFloats, 4);
+  pl.sg_shift = log2_int(nthreads);
+  pl.lds_floats = pl.plane_lds_floats;
+  pl.groups_per_channel = 1;
   const uintptr_t mask = 4 * elem_size - 1;       // 4-element vectors: 16 B (fp32) / 8 B (bf16)
   auto aligned = [mask](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
   pl.vec_ok = (W % 4 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
-  if (pl.vec_ok) {
-    // 2x4 pieces per row-pair, walked by groups of the next power of two of W/4 lanes
-    int gs = 1;
-    while (gs < W / 4) gs *= 2;
-    const int rows_per_pass = nthreads / gs;
-    pl.prefetch = rows_per_pass >= 1 && (pl.h[1] + rows_per_pass - 1) / rows_per_pass <= kFetchPasses;
-  }
   return pl;
+}
+
+// Completes a plan for the plane kernel: threads per plane, slots per workgroup, prefetch.
+inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
+  pl->sg_shift = tj1_sg_shift;
+  const int sg = 1 << pl->sg_shift;
+  const int slots = 256 / sg;
+  pl->lds_floats = pl->plane_lds_floats * slots;
+  const int ppw = sg < kWave ? kWave / sg : 1;
+  pl->groups_per_channel = (pl->B + ppw - 1) / ppw;
+  pl->prefetch = 0;
+  if (pl->vec_ok) {
+    const int gs = pow2_ceil(pl->W / 4);       // 2x4 pieces per row pair, one lane each
+    const int rows_per_pass = sg / gs;
+    pl->prefetch = rows_per_pass >= 1 && (pl->h[1] + rows_per_pass - 1) / rows_per_pass <= kFetchPasses;
+  }
 }
 
 // Batch chunking of the weight-gradient kernels: enough workgroups to fill 256 CUs a few
