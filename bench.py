@@ -263,8 +263,7 @@ def main():
                           "bytes_written": src.numel() * src.element_size(), "launches": args.warmup + args.steps}))
         return
 
-    main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup,
-                           per_kernel=not args.no_extra)
+    main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup, per_kernel=True)
     line = {
         "metric": "WTConv2d fwd+bwd images/s",
         "value": main_res["images_per_s"],

@@ -108,6 +108,10 @@ static int check_common(const char* fn, const wtconv_params* params, int B, int 
   return 0;
 }
 
+// Workgroups of the weight-gradient kernel assumed resident when chunking the batch (2 per
+// CU on 256 CUs).  A constant, so that workspace sizes do not depend on the device queried.
+constexpr int kWgradResident = 512;
+
 static size_t fold_floats(int C, int S, int L, int KK) { return static_cast<size_t>(C) * (1 + S * L) * KK + C; }
 
 static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float* fb, int C, int S, int L,
@@ -336,12 +340,11 @@ int wtconv_debug_phase_ticks(unsigned long long* out16, int reset) {
 #endif
 
 size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
-  (void)H; (void)W;
-  if (B <= 0 || C <= 0 || K <= 0 || levels <= 0) return 0;
+  if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     int bchunk, nchunk;
-    wgrad_chunks(B, C, &bchunk, &nchunk);
+    wgrad_chunks(B, C, wgrad_planes_per_iter(B, H, W, K, levels), kWgradResident, &bchunk, &nchunk);
     floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
   } else {
     floats = fold_floats(C, 4, levels, K * K);
@@ -381,7 +384,9 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  const Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr);
+  const int pb = wgrad_planes_per_iter(B, H, W, K, L);
+  Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
+  finish_wgrad_plan(&pl);
   if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
     return fail(WTCONV_E_UNSUPPORTED,
                 "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
@@ -391,7 +396,7 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   int bchunk, nchunk;
-  wgrad_chunks(B, C, &bchunk, &nchunk);
+  wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
   float* partial = static_cast<float*>(workspace);
   const int e = dtype == WTCONV_F32
                     ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)

@@ -23,6 +23,7 @@
 #define WT_WAIT_VMEM() do {} while (0)
 #define WT_CHUNK_FENCE() do {} while (0)
 #define WT_LAUNDER_UNIFORM_PTR(p) do {} while (0)
+#define WT_LAUNDER_LANE_INT(v) do {} while (0)
 typedef const float* wt_uniform_ptr;
 #else
 // Folded weights are read-only for the whole launch and indexed uniformly: the constant
@@ -56,6 +57,10 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 // are issued here (25 SGPRs live) instead of being hoisted out of the row loop all at once
 // (hundreds of SGPRs, spilled to VGPR lanes).
 #define WT_LAUNDER_UNIFORM_PTR(p) asm volatile("" : "+s"(p))
+// Makes a per-lane index opaque inside a loop body, so that the addresses derived from it
+// are recomputed per iteration (a few integer ops) instead of being hoisted out of the loop
+// into long-lived registers that end up spilled.
+#define WT_LAUNDER_LANE_INT(v) asm volatile("" : "+v"(v))
 #endif
 
 // Optional profiling aid (off in the product build): -DWT_PHASE_TIMING makes wave 0 of

@@ -45,6 +45,8 @@ struct Plan2D {
   int sg_shift;                // log2 of the threads that share one plane (4..8)
   int plane_lds_floats;        // LDS of one plane slot; lds_floats = slots * this
   int groups_per_channel;      // sg < 64: a wave holds 64/sg planes of one channel; number of such groups per channel
+  int pb;                      // weight-gradient kernel: planes of one channel stacked per iteration
+  int slot_shift;              //   log2 of the threads that load/analyse one of them
 };
 
 // ------------------------------------------------------------------ parameter folding
@@ -82,18 +84,20 @@ __global__ void fold_params_kernel(ParamTable p, int pdtype, float* __restrict__
 // element (r, col) sits at dst[(r + P) * str + col + P].
 template <typename T>
 __device__ __forceinline__ void load_plane(const T* __restrict__ src, float* __restrict__ dst,
-                                           int H, int W, int str, int P, int tid, int nthreads) {
+                                           int H, int W, int str, int P, int tid, int nthreads,
+                                           bool valid = true) {
   const int gsh = W <= 1 ? 0 : 32 - __clz(W - 1);
   const int rpp = nthreads >> gsh;
   if (rpp >= 1) {                      // lane groups of 2^gsh >= W lanes walk whole rows
     const int col = tid & ((1 << gsh) - 1);
     if (col >= W || (tid >> gsh) >= rpp) return;
-    for (int r = tid >> gsh; r < H; r += rpp) dst[(r + P) * str + col + P] = to_f32<T>(src[r * W + col]);
+    for (int r = tid >> gsh; r < H; r += rpp)
+      dst[(r + P) * str + col + P] = valid ? to_f32<T>(src[r * W + col]) : 0.f;
   } else {
     const int n = H * W;
     for (int e = tid; e < n; e += nthreads) {
       const int r = e / W, col = e - r * W;
-      dst[(r + P) * str + col + P] = to_f32<T>(src[e]);
+      dst[(r + P) * str + col + P] = valid ? to_f32<T>(src[e]) : 0.f;
     }
   }
 }
@@ -127,7 +131,7 @@ template <typename T>
 __device__ __forceinline__ void load_analysis1(const T* __restrict__ src, int H, int W,
                                                float* __restrict__ d0, int str0, int P0,
                                                float* __restrict__ d1, int str1, int pl1, int P1,
-                                               int tid, int nthreads) {
+                                               int tid, int nthreads, bool valid = true) {
   const int h1 = (H + 1) >> 1;
   const int nitem = W >> 2;                     // 4-column pieces per row
   const int gsh = group_shift(nitem);
@@ -135,10 +139,12 @@ __device__ __forceinline__ void load_analysis1(const T* __restrict__ src, int H,
   if (s >= nitem) return;
   const int c0 = 4 * s;
   for (int i = tid >> gsh; i < h1; i += nthreads >> gsh) {
-    float a[4], b[4] = {0.f, 0.f, 0.f, 0.f};
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
     const bool has_b = 2 * i + 1 < H;
-    load4<T>(src + (2 * i) * W + c0, a);
-    if (has_b) load4<T>(src + (2 * i + 1) * W + c0, b);
+    if (valid) {
+      load4<T>(src + (2 * i) * W + c0, a);
+      if (has_b) load4<T>(src + (2 * i + 1) * W + c0, b);
+    }
     float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -187,7 +193,7 @@ template <int NP>
 __device__ __forceinline__ void plane_commit(const float (&a)[NP][4], const float (&b)[NP][4], int H, int W,
                                              float* __restrict__ d0, int str0, int P0,
                                              float* __restrict__ d1, int str1, int pl1, int P1,
-                                             int tid, int nthreads) {
+                                             int tid, int nthreads, bool valid = true) {
   const int h1 = (H + 1) >> 1;
   const int nitem = W >> 2;
   const int gsh = group_shift(nitem);
@@ -199,20 +205,23 @@ __device__ __forceinline__ void plane_commit(const float (&a)[NP][4], const floa
     const int i = (tid >> gsh) + p * (nthreads >> gsh);
     if (i < h1) {
       const bool has_b = 2 * i + 1 < H;
-      float bb[4];
+      float aa[4], bb[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) bb[k] = has_b ? b[p][k] : 0.f;
+      for (int k = 0; k < 4; ++k) {      // a slot without a plane commits zeros
+        aa[k] = valid ? a[p][k] : 0.f;
+        bb[k] = (valid && has_b) ? b[p][k] : 0.f;
+      }
       float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        x0[k] = a[p][k];
+        x0[k] = aa[k];
         if (has_b) x0[str0 + k] = bb[k];
       }
       float* o = d1 + (i + P1) * str1 + 2 * s + P1;
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const float sac = a[p][2 * t] + bb[2 * t], sbd = a[p][2 * t + 1] + bb[2 * t + 1];
-        const float dac = a[p][2 * t] - bb[2 * t], dbd = a[p][2 * t + 1] - bb[2 * t + 1];
+        const float sac = aa[2 * t] + bb[2 * t], sbd = aa[2 * t + 1] + bb[2 * t + 1];
+        const float dac = aa[2 * t] - bb[2 * t], dbd = aa[2 * t + 1] - bb[2 * t + 1];
         o[t] = 0.5f * (sac + sbd);
         o[pl1 + t] = 0.5f * (dac + dbd);
         o[2 * pl1 + t] = 0.5f * (sac - sbd);
@@ -527,7 +536,7 @@ __global__ __launch_bounds__(256, 4) void wt2d_plane_kernel(const T* __restrict_
   const size_t plane_elems = static_cast<size_t>(pl.H) * pl.W;
   const int tid = threadIdx.x;
   const int sg = 1 << pl.sg_shift;
-  const int ltid = tid & (sg - 1);
+  int ltid = tid & (sg - 1);
   const int slot = tid >> pl.sg_shift;
   const int slots = blockDim.x >> pl.sg_shift;
   float* lds = lds_all + slot * pl.plane_lds_floats;
@@ -635,14 +644,61 @@ __device__ __forceinline__ void corr_strip(const float* __restrict__ a, int astr
 #pragma unroll
       for (int t = 0; t < TJ; ++t) acc[kh * K + kw] = fmaf(dy[t], row[t + kw], acc[kh * K + kw]);
     }
+    if (TJ > 1 && kh == K / 2 && K > 3) {   // two chunks per strip: at most (K+1)/2 rows in flight
+      pin_values(acc);
+      pin_values(dy);
+      WT_CHUNK_FENCE();
+    }
+  }
+  pin_values(acc);
+  WT_CHUNK_FENCE();
+}
+
+// Two vertically adjacent strips at once: the K+1 input rows they span are read once, row r
+// feeding kernel row r of the upper strip and kernel row r-1 of the lower one (a third
+// fewer LDS reads per FMA than two separate strips).
+template <int K, int TJ, int VW>
+__device__ __forceinline__ void corr_strip2(const float* __restrict__ a, int astr,
+                                            const float* __restrict__ gy0, const float* __restrict__ gy1,
+                                            float (&acc)[K * K]) {
+  constexpr int NR = pad_to(TJ + K - 1, VW);
+  float dy0[TJ], dy1[TJ];
+  lds_row<TJ, (TJ % 4 == 0) ? 4 : 1>(gy0, dy0);
+  lds_row<TJ, (TJ % 4 == 0) ? 4 : 1>(gy1, dy1);
+#pragma unroll
+  for (int r = 0; r < K + 1; ++r) {
+    float row[NR];
+    lds_row<NR, VW>(a + r * astr, row);
+    if (r < K) {
+#pragma unroll
+      for (int kw = 0; kw < K; ++kw) {
+#pragma unroll
+        for (int t = 0; t < TJ; ++t) acc[r * K + kw] = fmaf(dy0[t], row[t + kw], acc[r * K + kw]);
+      }
+    }
+    if (r >= 1) {
+#pragma unroll
+      for (int kw = 0; kw < K; ++kw) {
+#pragma unroll
+        for (int t = 0; t < TJ; ++t) acc[(r - 1) * K + kw] = fmaf(dy1[t], row[t + kw], acc[(r - 1) * K + kw]);
+      }
+    }
+    if (r == K / 2) {
+      pin_values(acc);
+      pin_values(dy0);
+      pin_values(dy1);
+      WT_CHUNK_FENCE();
+    }
   }
   pin_values(acc);
   WT_CHUNK_FENCE();
 }
 
 // Correlation sums of one sub-band plane of one level, walked by a single wave.
-// row0/row_step select the rows this wave owns (all rows: 0 / rows-per-pass).
-template <int K, int TJ, int VW>
+// pass_row0/pass_step select the passes this wave owns (all: 0 / 1).  PAIR: work items are
+// pairs of rows (the row below the last one must exist and hold zeros in G: it is the gap
+// row under every stacked plane).
+template <int K, int TJ, int VW, bool PAIR>
 __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr, const float* __restrict__ G,
                                            int gstr, int h, int w, int lane, int pass_row0, int pass_step,
                                            float (&acc)[K * K], float gmul, float& gsum) {
@@ -651,19 +707,30 @@ __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr
   const int strip = lane & ((1 << gsh) - 1);
   if (strip >= nstrip) return;
   const int j0 = strip * TJ;
-  const int rpp = kWave >> gsh;          // rows per pass of one wave (>= 1: nstrip <= 64)
-  for (int i = pass_row0 * rpp + (lane >> gsh); i < h; i += pass_step * rpp) {
-    const float* gy = G + i * gstr + j0;
+  const int rpp = kWave >> gsh;          // row items per pass of one wave (>= 1: nstrip <= 64)
+  if constexpr (PAIR) {
+    const int npair = (h + 1) >> 1;
+    for (int ip = pass_row0 * rpp + (lane >> gsh); ip < npair; ip += pass_step * rpp) {
+      const int i = 2 * ip;
+      const float* gy = G + i * gstr + j0;
 #pragma unroll
-    for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t], gsum);
-    corr_strip<K, TJ, VW>(A + i * astr + j0, astr, gy, acc);   // A already points R rows/cols up-left
+      for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t] + gy[gstr + t], gsum);
+      corr_strip2<K, TJ, VW>(A + i * astr + j0, astr, gy, gy + gstr, acc);
+    }
+  } else {
+    for (int i = pass_row0 * rpp + (lane >> gsh); i < h; i += pass_step * rpp) {
+      const float* gy = G + i * gstr + j0;
+#pragma unroll
+      for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t], gsum);
+      corr_strip<K, TJ, VW>(A + i * astr + j0, astr, gy, acc);   // A already points R rows/cols up-left
+    }
   }
 }
 
 constexpr int wgrad_sets(int L) { return L >= 4 ? 3 : (L >= 2 ? 2 : 1); }
 
 template <typename T, int K, int L, int TJ>
-__global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
+__global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
                                                          float* __restrict__ partial, Plan2D pl,
                                                          int B, int bchunk) {
   WT_SHARED_FLOATS(lds);
@@ -676,10 +743,20 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
   const int chunk = blockIdx.y;
   const int tid = threadIdx.x;
   const int wave = WT_UNIFORM(tid >> 6);
-  const int lane = tid & (kWave - 1);
+  int lane = tid & (kWave - 1);
   const int q = wave & 3;
   const bool role_a = wave < 4;
   const int P = pl.P;
+  // `pb` planes (same channel, consecutive batch items) are stacked vertically per
+  // iteration, separated by the P zero rows that already serve as halo: a correlation over
+  // the stack is the sum of the per-plane correlations.  Slot k of the stack is loaded and
+  // analysed by the threads with tid >> slot_shift == k.
+  const int pb = pl.pb;
+  int slot = tid >> pl.slot_shift;
+  const int nps = 1 << pl.slot_shift;
+  int ltid = tid & (nps - 1);
+  const bool has_slot = slot < pb;
+  const size_t plane_elems = static_cast<size_t>(pl.H) * pl.W;
 
   float acc[NSET][KK];
   float gsum = 0.f;
@@ -688,62 +765,104 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
 #pragma unroll
     for (int t = 0; t < KK; ++t) acc[s][t] = 0.f;
 
+  WT_TICK_INIT();
   zero_lds(lds, pl.lds_floats);
-  WT_LDS_BARRIER();
 
-  // pointers to the top-left corner of the conv window of element (0,0)
+  // slot-local bases: level l of slot k starts k*(h_l+P) rows below the top of the stack
+  auto a_slot = [&](int l) { return lds + pl.aoff[l] + slot * (pl.h[l] + P) * pl.astr[l]; };
+  auto g_slot = [&](int l) { return lds + pl.goff[l] + slot * (pl.h[l] + P) * pl.gstr[l]; };
+  // pointers to the top-left corner of the conv window of element (0,0) of the stack
   auto a_plane = [&](int l, int s) { return lds + pl.aoff[l] + s * pl.apl[l] + (P - R) * pl.astr[l] + (P - R); };
   auto g_plane = [&](int l, int s) { return lds + pl.goff[l] + s * pl.gpl[l]; };
+  auto rows = [&](int l) { return pb * (pl.h[l] + P) - P; };
 
-  const int b_end = (chunk + 1) * bchunk < B ? (chunk + 1) * bchunk : B;
-  for (int bv = chunk * bchunk; bv < b_end; ++bv) {
-    const int b = WT_UNIFORM(bv);
-    const size_t plane_off = (static_cast<size_t>(b) * pl.C + c) * pl.H * pl.W;
-    int l0 = 1;
-    if (pl.vec_ok) {
-      load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], P,
-                        lds + pl.aoff[1], pl.astr[1], pl.apl[1], P, tid, blockDim.x);
-      load_analysis1<T>(g + plane_off, pl.H, pl.W, lds + pl.goff[0], pl.gstr[0], 0,
-                        lds + pl.goff[1], pl.gstr[1], pl.gpl[1], 0, tid, blockDim.x);
-      l0 = 2;
+  const int b_begin = chunk * bchunk;
+  const int b_end = b_begin + bchunk < B ? b_begin + bchunk : B;
+  float xa[1][4], xb[1][4], ga[1][4], gb[1][4];
+  if (pl.prefetch && has_slot) {
+    const bool valid = b_begin + slot < b_end;
+    const size_t off = (static_cast<size_t>(valid ? b_begin + slot : b_begin) * pl.C + c) * plane_elems;
+    plane_fetch<T, 1>(x + off, pl.H, pl.W, ltid, nps, xa, xb);
+    plane_fetch<T, 1>(g + off, pl.H, pl.W, ltid, nps, ga, gb);
+  }
+  WT_LDS_BARRIER();
+
+  for (int bv = b_begin; bv < b_end; bv += pb) {
+    const int b0 = WT_UNIFORM(bv);
+    WT_LAUNDER_LANE_INT(slot);
+    WT_LAUNDER_LANE_INT(ltid);
+    WT_LAUNDER_LANE_INT(lane);
+    const bool valid = has_slot && b0 + slot < b_end;
+    const size_t plane_off = (static_cast<size_t>(valid ? b0 + slot : b0) * pl.C + c) * plane_elems;
+    int l0 = 2;
+    if (pl.prefetch) {
+      if (has_slot) {
+        plane_commit<1>(xa, xb, pl.H, pl.W, a_slot(0), pl.astr[0], P, a_slot(1), pl.astr[1], pl.apl[1], P, ltid, nps,
+                        valid);
+        plane_commit<1>(ga, gb, pl.H, pl.W, g_slot(0), pl.gstr[0], 0, g_slot(1), pl.gstr[1], pl.gpl[1], 0, ltid, nps,
+                        valid);
+      }
+    } else if (pl.vec_ok) {
+      if (has_slot) {
+        load_analysis1<T>(x + plane_off, pl.H, pl.W, a_slot(0), pl.astr[0], P, a_slot(1), pl.astr[1], pl.apl[1], P,
+                          ltid, nps, valid);
+        load_analysis1<T>(g + plane_off, pl.H, pl.W, g_slot(0), pl.gstr[0], 0, g_slot(1), pl.gstr[1], pl.gpl[1], 0,
+                          ltid, nps, valid);
+      }
     } else {
-      load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], P, tid, blockDim.x);
-      load_plane<T>(g + plane_off, lds + pl.goff[0], pl.H, pl.W, pl.gstr[0], 0, tid, blockDim.x);
+      if (has_slot) {
+        load_plane<T>(x + plane_off, a_slot(0), pl.H, pl.W, pl.astr[0], P, ltid, nps, valid);
+        load_plane<T>(g + plane_off, g_slot(0), pl.H, pl.W, pl.gstr[0], 0, ltid, nps, valid);
+      }
+      l0 = 1;
     }
     WT_LDS_BARRIER();
+    WT_TICK(8);
+    if (pl.prefetch && has_slot && b0 + pb < b_end) {
+      const bool nvalid = b0 + pb + slot < b_end;
+      const size_t off = (static_cast<size_t>(nvalid ? b0 + pb + slot : b0) * pl.C + c) * plane_elems;
+      plane_fetch<T, 1>(x + off, pl.H, pl.W, ltid, nps, xa, xb);   // an absent plane re-reads plane b0:
+      plane_fetch<T, 1>(g + off, pl.H, pl.W, ltid, nps, ga, gb);   //   zeroed at commit
+    }
     for (int lv = l0; lv <= L; ++lv) {
       const int l = WT_UNIFORM(lv);
-      analysis_level(lds + pl.aoff[l - 1], pl.astr[l - 1], P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], P,
-                     pl.h[l], pl.w[l], tid, blockDim.x);
-      analysis_level(lds + pl.goff[l - 1], pl.gstr[l - 1], 0, lds + pl.goff[l], pl.gstr[l], pl.gpl[l], 0,
-                     pl.h[l], pl.w[l], tid, blockDim.x);
+      if (has_slot) {
+        analysis_level(a_slot(l - 1), pl.astr[l - 1], P, a_slot(l), pl.astr[l], pl.apl[l], P, pl.h[l], pl.w[l],
+                       ltid, nps);
+        analysis_level(g_slot(l - 1), pl.gstr[l - 1], 0, g_slot(l), pl.gstr[l], pl.gpl[l], 0, pl.h[l], pl.w[l],
+                       ltid, nps);
+      }
       WT_LDS_BARRIER();
     }
+    WT_TICK(9);
     // Both roles run the same code on different planes (one code path keeps a single
-    // register set for the sums): level index per set, -1 = base conv, 0 = nothing.
+    // register set for the sums).
     {
       const int l = role_a ? 0 : 1;            // set 0, strips of TJ: base conv rows (A) / level 1 (B)
-      corr_level<K, TJ, VW>(a_plane(l, role_a ? 0 : q), pl.astr[l], g_plane(l, role_a ? 0 : q), pl.gstr[l],
-                            pl.h[l], pl.w[l], lane, role_a ? q : 0, role_a ? 4 : 1, acc[0], role_a ? 1.f : 0.f,
+      corr_level<K, TJ, VW, true>(a_plane(l, role_a ? 0 : q), pl.astr[l], g_plane(l, role_a ? 0 : q), pl.gstr[l],
+                            rows(l), pl.w[l], lane, role_a ? q : 0, role_a ? 4 : 1, acc[0], role_a ? 1.f : 0.f,
                             gsum);
     }
+    WT_TICK(10);
     if constexpr (NSET >= 2) {                 // set 1, single coefficients: level 3 (A) / level 2 (B)
       const int l = role_a ? 3 : 2;
       if (l <= L) {
         float unused = 0.f;
-        corr_level<K, 1, 1>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], pl.h[l], pl.w[l], lane, 0, 1,
-                            acc[1], 0.f, unused);
+        corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0, 1,
+                                   acc[1], 0.f, unused);
       }
     }
     if constexpr (NSET >= 3) {                 // set 2: level 5 (A) / level 4 (B)
       const int l = role_a ? 5 : 4;
       if (l <= L) {
         float unused = 0.f;
-        corr_level<K, 1, 1>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], pl.h[l], pl.w[l], lane, 0, 1,
-                            acc[2], 0.f, unused);
+        corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0, 1,
+                                   acc[2], 0.f, unused);
       }
     }
+    WT_TICK(11);
     WT_LDS_BARRIER();
+    WT_TICK(12);
   }
 
   // cross-lane reduction, then cross-wave through LDS (pyramid buffers are dead now)
@@ -761,6 +880,7 @@ __global__ __launch_bounds__(512) void wt2d_wgrad_kernel(const T* __restrict__ x
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
   WT_LDS_BARRIER();
+  WT_TICK(13);
   float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * (NF * KK + 1);
   for (int o = tid; o < NF * KK + 1; o += blockDim.x) {
     float v = 0.f;

@@ -40,7 +40,7 @@ inline void choose_plane_shape(int h1, int w1, int* tj1, int* sg_shift) {
 // with_grad_pyramid adds the padded pyramid of grad_out used by the weight-gradient kernel
 // (and drops the Z buffers it does not need).
 inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
-                          size_t elem_size, const void* p0, const void* p1, const void* p2) {
+                          size_t elem_size, const void* p0, const void* p1, const void* p2, int pb = 1) {
   Plan2D pl = {};
   pl.B = B; pl.C = C; pl.H = H; pl.W = W; pl.L = L;
   pl.nplanes = B * C;
@@ -52,7 +52,7 @@ inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_gr
   int off = 0;            // start of the zero gap above the next plane
   for (int l = 0; l <= L; ++l) {
     pl.astr[l] = round_up(pl.w[l] + 2 * pl.P, 4);
-    pl.apl[l] = (pl.h[l] + pl.P) * pl.astr[l];
+    pl.apl[l] = pb * (pl.h[l] + pl.P) * pl.astr[l];        // pb planes stacked, P shared zero rows between them
     if (l > 0) off += pl.P * (pl.astr[l - 1] - pl.astr[l]);   // the gap keeps the wider stride of the level above
     pl.aoff[l] = off;
     off += pl.apl[l] * (l == 0 ? 1 : 4);
@@ -67,13 +67,15 @@ inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_gr
   } else {
     for (int l = 0; l <= L; ++l) {
       pl.gstr[l] = round_up(pl.w[l] + 1, 4);
-      pl.gpl[l] = pl.gstr[l] * (pl.h[l] + 1);
+      pl.gpl[l] = pb * (pl.h[l] + pl.P) * pl.gstr[l];      // same row pitch as the x pyramid
       pl.goff[l] = off;
       off += pl.gpl[l] * (l == 0 ? 1 : 4);
     }
   }
   pl.plane_lds_floats = round_up(off + kLdsSlackFloats, 4);
   pl.sg_shift = log2_int(nthreads);
+  pl.pb = pb;
+  pl.slot_shift = log2_int(nthreads);
   pl.lds_floats = pl.plane_lds_floats;
   pl.groups_per_channel = 1;
   const uintptr_t mask = 4 * elem_size - 1;       // 4-element vectors: 16 B (fp32) / 8 B (bf16)
@@ -98,13 +100,52 @@ inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
   }
 }
 
-// Batch chunking of the weight-gradient kernels: enough workgroups to fill 256 CUs a few
-// times over, long enough chunks to amortise the end-of-chunk reduction.
-inline void wgrad_chunks(int B, int C, int* bchunk, int* nchunk) {
-  int want = (1536 + C - 1) / C;          // workgroups per channel
-  if (want < 1) want = 1;
-  if (want > B) want = B;
-  int bc = (B + want - 1) / want;
+// Planes per iteration of the weight-gradient kernel: as many as fill one pass of the four
+// base-conv waves over the rows of the stack, within the LDS budget.
+inline int wgrad_planes_per_iter(int B, int H, int W, int K, int L) {
+  const int P = K / 2 > 1 ? K / 2 : 1;
+  const int gs = pow2_ceil((W + kTJW - 1) / kTJW);
+  const int rows_per_pass = gs <= 64 ? 4 * (64 / gs) : 4;
+  int pb = rows_per_pass / (H + P);
+  if (pb < 1) pb = 1;
+  if (pb > 16) pb = 16;
+  if (pb > B) pb = B;
+  while (pb > 1) {
+    const Plan2D t = make_plan2d(B, 1, H, W, K, L, true, 512, 4, nullptr, nullptr, nullptr, pb);
+    if (static_cast<size_t>(t.plane_lds_floats) * 4 <= 80 * 1024) break;
+    --pb;
+  }
+  return pb;
+}
+
+// Completes a plan for the weight-gradient kernel: threads per stacked plane, prefetch.
+inline void finish_wgrad_plan(Plan2D* pl) {
+  const int slots = pow2_ceil(pl->pb);
+  pl->slot_shift = log2_int(512 / slots);
+  const int nps = 512 / slots;
+  pl->prefetch = 0;
+  if (pl->vec_ok) {
+    const int gs = pow2_ceil(pl->W / 4);
+    pl->prefetch = nps / gs >= pl->h[1];       // one 2x4 piece per thread covers the plane
+  }
+}
+
+// Batch chunking of the 2-D weight-gradient kernel; a chunk is a whole number of
+// iterations of `pb` planes.  `resident` = workgroups the device holds at once.
+inline void wgrad_chunks(int B, int C, int pb, int resident, int* bchunk, int* nchunk) {
+  // Chunks per channel n: C*n workgroups run in ceil(C*n/resident) rounds.  Every workgroup
+  // pays LDS zeroing, a cold first fetch and the final reduction once, so score = fill of
+  // the rounds minus 5 % per round, and the best n wins (ties: the smaller).
+  const int iters = (B + pb - 1) / pb;           // iterations available per channel
+  int best_n = 1;
+  double best = -1.0;
+  for (int n = 1; n <= iters && n <= 64; ++n) {
+    const int wgs = C * n;
+    const int rounds = (wgs + resident - 1) / resident;
+    const double score = static_cast<double>(wgs) / (static_cast<double>(rounds) * resident) - 0.05 * rounds;
+    if (score > best + 1e-9) { best = score; best_n = n; }
+  }
+  int bc = (iters + best_n - 1) / best_n * pb;
   if (bc < 1) bc = 1;
   *bchunk = bc;
   *nchunk = (B + bc - 1) / bc;
