@@ -73,6 +73,8 @@ def _built():
     (1, 1, 12, 20, 7, 1, True),     # K = 7, single level
     (2, 1, 6, 10, 1, 2, True),      # K = 1 (no conv halo)
     (1, 1, 28, 28, 5, 5, True),     # five levels: 28 14 7 4 2 1
+    (5, 3, 7, 7, 5, 2, True),       # several small planes per workgroup / per wave, ragged batch tail
+    (3, 2, 14, 14, 3, 2, True),     # 16 threads per plane, stacked planes in the weight-gradient kernel
 ])
 def test_emulated_2d_fp32(B, C, H, W, K, L, bias):
     x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias)

@@ -235,8 +235,8 @@ static int run_tile1d(const void* x, void* out, const float* fw, const float* fb
   auto kern = wt1d_tile_kernel<T, K, kTJ1D>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
-  WT_LAUNCH(kern, dim3(pl.ntiles, B * pl.C), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out),
-            fw, fb, pl);
+  WT_LAUNCH(kern, dim3(pl.ntiles, B * pl.C), dim3(kBlock1D), lds, stream, static_cast<const T*>(x),
+            static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt1d_tile_kernel");
 }
 
@@ -258,8 +258,8 @@ static int run_wgrad1d(const void* x, const void* g, float* partial, const Plan1
   auto kern = wt1d_wgrad_kernel<T, K, L, kTJ1D>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
-  WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<const T*>(g),
-            partial, pl, B, per_chunk);
+  WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(kBlock1D), lds, stream, static_cast<const T*>(x),
+            static_cast<const T*>(g), partial, pl, B, per_chunk);
   return check_launch("wt1d_wgrad_kernel");
 }
 

@@ -35,6 +35,8 @@ struct Plan1D {
 
 constexpr float kInvSqrt2 = 0.70710678118654752440f;
 
+constexpr int kBlock1D = 256;   // threads per workgroup of the 1-D kernels
+
 // Stage samples [t0 - halo, t0 + T + halo) of one row; zero outside [0, N).
 template <typename T>
 __device__ __forceinline__ void load_row_tile(const T* __restrict__ row, float* __restrict__ dst,
@@ -125,10 +127,10 @@ __device__ __forceinline__ void store_run(T* __restrict__ dst, const float (&v)[
   }
 }
 
-// Forward / input-gradient kernel.  grid = (ntiles, B*C), block = 256.
+// Forward / input-gradient kernel.  grid = (ntiles, B*C), block = kBlock1D.
 // TJ level-l coefficients (2*TJ outputs of the level below) per work item; TJ = 4.
 template <typename T, int K, int TJ>
-__global__ __launch_bounds__(256) void wt1d_tile_kernel(const T* __restrict__ x, T* __restrict__ out,
+__global__ __launch_bounds__(kBlock1D) void wt1d_tile_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                         const float* __restrict__ fw,
                                                         const float* __restrict__ fb, Plan1D pl) {
   WT_SHARED_FLOATS(lds);
@@ -143,11 +145,11 @@ __global__ __launch_bounds__(256) void wt1d_tile_kernel(const T* __restrict__ x,
   T* orow = out + static_cast<size_t>(row) * pl.N;
 
   load_row_tile<T>(xrow, lds + pl.aoff[0], pl.N, t0 - pl.hal[0], pl.tl[0] + 2 * pl.hal[0], pl.vec_ok != 0);
-  __syncthreads();
+  WT_LDS_BARRIER();
   for (int l = 1; l <= pl.L; ++l) {
     analysis1d_level(lds + pl.aoff[l - 1], lds + pl.aoff[l], pl.apl[l], pl.tl[l] + 2 * pl.hal[l],
                      threadIdx.x, blockDim.x);
-    __syncthreads();
+    WT_LDS_BARRIER();
   }
   for (int l = pl.L; l >= 2; --l) {
     const int tl = pl.tl[l];
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(256) void wt1d_tile_kernel(const T* __restrict__ x,
         }
       }
     }
-    __syncthreads();
+    WT_LDS_BARRIER();
   }
   {
     const int tl = pl.tl[1];
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(256) void wt1d_tile_kernel(const T* __restrict__ x,
   }
 }
 
-// Parameter gradients, first stage.  grid = (C, nchunk), block = 256.  A workgroup walks
+// Parameter gradients, first stage.  grid = (C, nchunk), block = kBlock1D.  A workgroup walks
 // `per_chunk` (row, tile) pairs of one channel, every thread keeps K sums per filter in
 // registers; reduction and output layout as in the 2-D kernel:
 //   partial[chunk][c][ (1 + 2L) * K + 1 ]
@@ -234,7 +236,7 @@ __device__ __forceinline__ void corr1_strip(const float* __restrict__ a, const f
 }
 
 template <typename T, int K, int L, int TJ>
-__global__ __launch_bounds__(256) void wt1d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
+__global__ __launch_bounds__(kBlock1D) void wt1d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
                                                          float* __restrict__ partial, Plan1D pl, int B,
                                                          int per_chunk) {
   WT_SHARED_FLOATS(lds);
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(256) void wt1d_wgrad_kernel(const T* __restrict__ x
     for (int k = 0; k < K; ++k) { accl[l][0][k] = 0.f; accl[l][1][k] = 0.f; }
 
   for (int v = tid; v < pl.lds_floats; v += blockDim.x) lds[v] = 0.f;
-  __syncthreads();
+  WT_LDS_BARRIER();
 
   const int total = B * pl.ntiles;
   const int w_end = (chunk + 1) * per_chunk < total ? (chunk + 1) * per_chunk : total;
@@ -265,12 +267,12 @@ __global__ __launch_bounds__(256) void wt1d_wgrad_kernel(const T* __restrict__ x
     const size_t roff = (static_cast<size_t>(b) * pl.C + c) * pl.N;
     load_row_tile<T>(x + roff, lds + pl.aoff[0], pl.N, t0 - pl.hal[0], pl.tl[0] + 2 * pl.hal[0], pl.vec_ok != 0);
     load_row_tile<T>(g + roff, lds + pl.goff[0], pl.N, t0, pl.tl[0], pl.vec_ok != 0);
-    __syncthreads();
+    WT_LDS_BARRIER();
 #pragma unroll
     for (int l = 1; l <= L; ++l) {
       analysis1d_level(lds + pl.aoff[l - 1], lds + pl.aoff[l], pl.apl[l], pl.tl[l] + 2 * pl.hal[l], tid, blockDim.x);
       analysis1d_level(lds + pl.goff[l - 1], lds + pl.goff[l], pl.gpl[l], pl.tl[l], tid, blockDim.x);
-      __syncthreads();
+      WT_LDS_BARRIER();
     }
     {
       const int items = (pl.tl[0] + TJ - 1) / TJ;
@@ -294,11 +296,11 @@ __global__ __launch_bounds__(256) void wt1d_wgrad_kernel(const T* __restrict__ x
         corr1_strip<K, TJ>(A + pl.apl[l] + i0 + pl.hal[l] - R, G + pl.gpl[l] + i0, accl[l - 1][1]);
       }
     }
-    __syncthreads();
+    WT_LDS_BARRIER();
   }
 
   constexpr int NRED = NF * K + 1;
-  float* red = lds;   // [4 waves][NRED]
+  float* red = lds;   // [waves][NRED]
   const int wave = tid >> 6, lane = tid & (kWave - 1);
 #pragma unroll
   for (int k = 0; k < K; ++k) {
@@ -318,10 +320,14 @@ __global__ __launch_bounds__(256) void wt1d_wgrad_kernel(const T* __restrict__ x
     const float v = wave_sum(gsum);
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
-  __syncthreads();
+  WT_LDS_BARRIER();
   float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * NRED;
-  for (int o = tid; o < NRED; o += blockDim.x)
-    dst[o] = red[o] + red[NRED + o] + red[2 * NRED + o] + red[3 * NRED + o];
+  const int nwaves = blockDim.x >> 6;
+  for (int o = tid; o < NRED; o += blockDim.x) {
+    float v = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) v += red[wv * NRED + o];
+    dst[o] = v;
+  }
 }
 
 }  // namespace wt
