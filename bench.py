@@ -22,6 +22,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 VALU_PEAK_TFLOPS = 78.6         # fp32 vector FMA without packed-FP32 code generation
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per
+# run), scaled by what a plain device copy of one activation tensor reads on the same
+# counters (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); see profiles/wt2d_stage1_fp32_hbm_traffic.txt.
+MEASURED_TRAFFIC_BYTES = {
+    ("stage1", "fp32", "wt2d_plane_kernel"): (151069 + 158737) * 1024,
+    ("stage1", "fp32", "wt2d_wgrad_kernel"): (301324 + 623) * 1024,
+}
+
 WORKLOADS = {
     # name: (C, H, W, K, L, batch)
     "stage1": (96, 56, 56, 5, 3, 128),
@@ -281,10 +289,18 @@ def main():
     }
     if "kernels" in main_res:
         line["kernels"] = main_res["kernels"]
-        name, k = max(main_res["kernels"].items(), key=lambda kv: kv[1]["avg_ms"])
+        # dominant kernel = most time per step: wt2d_plane_kernel runs twice (forward and
+        # input gradient); its forward launches are the ones reported
+        ks = main_res["kernels"]
+        plane_total = ks["wt2d_plane_kernel(forward)"]["avg_ms"] + ks["wt2d_plane_kernel(backward_input)"]["avg_ms"]
+        name = "wt2d_plane_kernel(forward)" if plane_total >= ks["wt2d_wgrad_kernel"]["avg_ms"] else "wt2d_wgrad_kernel"
+        k = ks[name]
         line["roofline"] = {"bound": "hbm", "kernel": name, "achieved": k["GBps"], "peak": HBM_PEAK_GBPS,
-                            "unit": "GB/s", "frac": k["GBps"] / HBM_PEAK_GBPS, "traffic": None,
-                            "avg_launch_ms": k["avg_ms"], "algorithmic_bytes_per_launch": k["algorithmic_bytes"]}
+                            "unit": "GB/s", "frac": k["GBps"] / HBM_PEAK_GBPS,
+                            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype, name.split("(")[0])),
+                            "avg_launch_ms": k["avg_ms"], "algorithmic_bytes_per_launch": k["algorithmic_bytes"],
+                            "valu_frac": 2 * mac_per_pixel(K, L) * B * C * H * W / (k["avg_ms"] * 1e-3) / 1e12
+                                         / VALU_PEAK_TFLOPS}
     else:
         line["roofline"] = {"bound": "hbm", "kernel": "whole step", "achieved": main_res["step_GBps"],
                             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": main_res["step_frac_hbm"], "traffic": None}
