@@ -132,11 +132,11 @@ static int run_plane2d(const void* x, void* out, const float* fw, const float* f
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   const int sg = 1 << pl.sg_shift;
-  const int slots = 256 / sg;
+  const int slots = pl.block / sg;
   const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
-  int nwg = compute_units() * resident_per_cu(kern, 256, lds);
+  int nwg = compute_units() * resident_per_cu(kern, pl.block, lds);
   if (nwg > nunits) nwg = nunits;
-  WT_LAUNCH(kern, dim3(nwg), dim3(256), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
+  WT_LAUNCH(kern, dim3(nwg), dim3(pl.block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
 }
 

@@ -45,6 +45,8 @@ struct Plan2D {
   int sg_shift;                // log2 of the threads that share one plane (4..8)
   int plane_lds_floats;        // LDS of one plane slot; lds_floats = slots * this
   int groups_per_channel;      // sg < 64: a wave holds 64/sg planes of one channel; number of such groups per channel
+  int fuse;                    // deepest analysis level produced from registers at commit (1..3)
+  int block;                   // plane kernel: threads per workgroup (256, or 512 = two whole-workgroup planes)
   int pb;                      // weight-gradient kernel: planes of one channel stacked per iteration
   int slot_shift;              //   log2 of the threads that load/analyse one of them
 };
@@ -226,6 +228,90 @@ __device__ __forceinline__ void plane_commit(const float (&a)[NP][4], const floa
         o[pl1 + t] = 0.5f * (dac + dbd);
         o[2 * pl1 + t] = 0.5f * (sac - sbd);
         o[3 * pl1 + t] = 0.5f * (dac - dbd);
+      }
+    }
+  }
+}
+
+// plane_commit that also produces levels 2 (and 3) straight from the registers: with the
+// lane layout (row-pair i, piece s) = (lane >> gsh, lane & (2^gsh - 1)) the 2x2 block of
+// level-1 LL values behind a level-2 coefficient sits in lanes i and i^1, and the level-2
+// block behind a level-3 coefficient in lanes (i, s), (i, s^1), (i^2, s), (i^2, s^1) of the
+// same wavefront, so wavefront shuffles replace two LDS round trips and two barriers per
+// plane.  Needs 2^gsh <= 16 lanes per row (so that 4 row-pairs share a wave) and every lane
+// of the wave in the call; lanes without a piece contribute zeros, which is also the
+// zero padding of odd sizes.  `fuse` = deepest level produced (2 or 3).
+template <int NP>
+__device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], const float (&b)[NP][4], int H, int W,
+                                                   float* __restrict__ d0, int str0, int P0,
+                                                   float* __restrict__ d1, int str1, int pl1,
+                                                   float* __restrict__ d2, int str2, int pl2,
+                                                   float* __restrict__ d3, int str3, int pl3, int P1,
+                                                   int fuse, int tid, int nthreads) {
+  const int h1 = (H + 1) >> 1;
+  const int nitem = W >> 2;
+  const int gsh = group_shift(nitem);
+  const int s = tid & ((1 << gsh) - 1);
+  const int c0 = 4 * s;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int i = (tid >> gsh) + p * (nthreads >> gsh);
+    const bool valid = s < nitem && i < h1;
+    const bool has_b = 2 * i + 1 < H;
+    float aa[4], bb[4], ll1[2];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      aa[k] = valid ? a[p][k] : 0.f;
+      bb[k] = (valid && has_b) ? b[p][k] : 0.f;
+    }
+    if (valid) {
+      float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x0[k] = aa[k];
+        if (has_b) x0[str0 + k] = bb[k];
+      }
+    }
+    float* o1 = d1 + (i + P1) * str1 + 2 * s + P1;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const float sac = aa[2 * t] + bb[2 * t], sbd = aa[2 * t + 1] + bb[2 * t + 1];
+      const float dac = aa[2 * t] - bb[2 * t], dbd = aa[2 * t + 1] - bb[2 * t + 1];
+      ll1[t] = 0.5f * (sac + sbd);
+      if (valid) {
+        o1[t] = ll1[t];
+        o1[pl1 + t] = 0.5f * (dac + dbd);
+        o1[2 * pl1 + t] = 0.5f * (sac - sbd);
+        o1[3 * pl1 + t] = 0.5f * (dac - dbd);
+      }
+    }
+    // level 2: rows i (even) and i+1 of level 1
+    const float bot0 = __shfl_xor(ll1[0], 1 << gsh, kWave);
+    const float bot1 = __shfl_xor(ll1[1], 1 << gsh, kWave);
+    const bool own2 = valid && (i & 1) == 0;
+    float ll2;
+    {
+      const float sac = ll1[0] + bot0, sbd = ll1[1] + bot1, dac = ll1[0] - bot0, dbd = ll1[1] - bot1;
+      ll2 = own2 ? 0.5f * (sac + sbd) : 0.f;
+      if (own2) {
+        float* o2 = d2 + ((i >> 1) + P1) * str2 + s + P1;
+        o2[0] = ll2;
+        o2[pl2] = 0.5f * (dac + dbd);
+        o2[2 * pl2] = 0.5f * (sac - sbd);
+        o2[3 * pl2] = 0.5f * (dac - dbd);
+      }
+    }
+    if (fuse >= 3) {   // level 3: level-2 positions (i/2, s), (i/2, s+1), (i/2+1, s), (i/2+1, s+1)
+      const float right = __shfl_xor(ll2, 1, kWave);
+      const float down = __shfl_xor(ll2, 2 << gsh, kWave);
+      const float diag = __shfl_xor(right, 2 << gsh, kWave);
+      if (valid && (i & 3) == 0 && (s & 1) == 0) {
+        const float sac = ll2 + down, sbd = right + diag, dac = ll2 - down, dbd = right - diag;
+        float* o3 = d3 + ((i >> 2) + P1) * str3 + (s >> 1) + P1;
+        o3[0] = 0.5f * (sac + sbd);
+        o3[pl3] = 0.5f * (dac + dbd);
+        o3[2 * pl3] = 0.5f * (sac - sbd);
+        o3[3 * pl3] = 0.5f * (dac - dbd);
       }
     }
   }
@@ -520,14 +606,15 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 }
 
 // Forward (and, with flipped folded weights and zero fb, input-gradient) kernel.
-// Persistent: grid.x = min(work units, resident workgroups), block = 256 threads.
-// 2^sg_shift threads share a plane, so a workgroup holds 256 >> sg_shift planes, each in its
-// own LDS slot (small planes: up to 16 per workgroup).  When a plane takes less than a wave,
+// Persistent: grid.x = min(work units, resident workgroups), block = 256 or 512 threads.
+// 2^sg_shift threads share a plane, so a workgroup holds blockDim >> sg_shift planes, each in
+// its own LDS slot (small planes: up to 16 per workgroup; planes that take 256 threads run
+// two to a workgroup, which halves the barrier-bound cost of their small coarse levels).  When a plane takes less than a wave,
 // the planes of one wave are the same channel of consecutive batch items, so the folded
 // weights stay wave-uniform (SGPRs).  The zero halos written once stay valid for every plane
 // (only interiors are rewritten).
 template <typename T, int K, int TJ1, int TJC>
-__global__ __launch_bounds__(256, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
+__global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                          const float* __restrict__ fw,
                                                          const float* __restrict__ fb, Plan2D pl) {
   WT_SHARED_FLOATS(lds_all);
@@ -795,7 +882,15 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     const bool valid = has_slot && b0 + slot < b_end;
     const size_t plane_off = (static_cast<size_t>(valid ? b0 + slot : b0) * pl.C + c) * plane_elems;
     int l0 = 2;
-    if (pl.prefetch) {
+    if (pl.prefetch && pl.fuse >= 2) {      // one plane per iteration: every lane takes part
+      plane_commit_fused<1>(xa, xb, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], P, lds + pl.aoff[1], pl.astr[1],
+                            pl.apl[1], lds + pl.aoff[2], pl.astr[2], pl.apl[2], lds + pl.aoff[pl.fuse],
+                            pl.astr[pl.fuse], pl.apl[pl.fuse], P, pl.fuse, tid, blockDim.x);
+      plane_commit_fused<1>(ga, gb, pl.H, pl.W, lds + pl.goff[0], pl.gstr[0], 0, lds + pl.goff[1], pl.gstr[1],
+                            pl.gpl[1], lds + pl.goff[2], pl.gstr[2], pl.gpl[2], lds + pl.goff[pl.fuse],
+                            pl.gstr[pl.fuse], pl.gpl[pl.fuse], 0, pl.fuse, tid, blockDim.x);
+      l0 = pl.fuse + 1;
+    } else if (pl.prefetch) {
       if (has_slot) {
         plane_commit<1>(xa, xb, pl.H, pl.W, a_slot(0), pl.astr[0], P, a_slot(1), pl.astr[1], pl.apl[1], P, ltid, nps,
                         valid);

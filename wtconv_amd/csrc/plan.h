@@ -88,15 +88,19 @@ inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_gr
 inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
   pl->sg_shift = tj1_sg_shift;
   const int sg = 1 << pl->sg_shift;
-  const int slots = 256 / sg;
+  pl->block = 256;   // (two whole planes per 512-thread workgroup measured slower: lockstep phases)
+  const int slots = pl->block / sg;
   pl->lds_floats = pl->plane_lds_floats * slots;
   const int ppw = sg < kWave ? kWave / sg : 1;
   pl->groups_per_channel = (pl->B + ppw - 1) / ppw;
   pl->prefetch = 0;
+  pl->fuse = 1;
   if (pl->vec_ok) {
     const int gs = pow2_ceil(pl->W / 4);       // 2x4 pieces per row pair, one lane each
     const int rows_per_pass = sg / gs;
     pl->prefetch = rows_per_pass >= 1 && (pl->h[1] + rows_per_pass - 1) / rows_per_pass <= kFetchPasses;
+    (void)gs;   // (measured: the fused commit does not pay in the plane kernel; it stays on in the
+                //  weight-gradient kernel, which builds two pyramids per plane)
   }
 }
 
@@ -124,9 +128,11 @@ inline void finish_wgrad_plan(Plan2D* pl) {
   pl->slot_shift = log2_int(512 / slots);
   const int nps = 512 / slots;
   pl->prefetch = 0;
+  pl->fuse = 1;
   if (pl->vec_ok) {
     const int gs = pow2_ceil(pl->W / 4);
     pl->prefetch = nps / gs >= pl->h[1];       // one 2x4 piece per thread covers the plane
+    if (pl->prefetch && pl->pb == 1 && gs <= 16 && pl->L >= 2) pl->fuse = pl->L >= 3 ? 3 : 2;
   }
 }
 
