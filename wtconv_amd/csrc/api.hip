@@ -125,10 +125,10 @@ static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float
 }
 
 // ---- 2-D dispatch over (dtype, K, level-1 strip width) -------------------------------
-template <typename T, int K, int TJ1>
-static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
-                       hipStream_t stream) {
-  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC>;
+template <typename T, int K, int TJ1, int MODE>
+static int run_plane2d_mode(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
+                            hipStream_t stream) {
+  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC, MODE>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   const int sg = 1 << pl.sg_shift;
@@ -138,6 +138,14 @@ static int run_plane2d(const void* x, void* out, const float* fw, const float* f
   if (nwg > nunits) nwg = nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(pl.block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
+}
+
+template <typename T, int K, int TJ1>
+static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
+                       hipStream_t stream) {
+  if (pl.prefetch) return run_plane2d_mode<T, K, TJ1, 0>(x, out, fw, fb, pl, stream);
+  if (pl.vec_ok) return run_plane2d_mode<T, K, TJ1, 1>(x, out, fw, fb, pl, stream);
+  return run_plane2d_mode<T, K, TJ1, 2>(x, out, fw, fb, pl, stream);
 }
 
 template <typename T, int K>

@@ -613,7 +613,10 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 // the planes of one wave are the same channel of consecutive batch items, so the folded
 // weights stay wave-uniform (SGPRs).  The zero halos written once stay valid for every plane
 // (only interiors are rewritten).
-template <typename T, int K, int TJ1, int TJC>
+// MODE selects the loader at compile time (0: register prefetch of the next plane, 1: fused
+// vector load without prefetch, 2: element-wise load), so that the hot variant does not carry
+// the registers of the others.
+template <typename T, int K, int TJ1, int TJC, int MODE>
 __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                          const float* __restrict__ fw,
                                                          const float* __restrict__ fb, Plan2D pl) {
@@ -652,7 +655,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   {
     int p0, c0;
     locate(blockIdx.x, p0, c0);
-    if (pl.prefetch && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
+    if (MODE == 0 && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
   }
   WT_LDS_BARRIER();
   WT_TICK(0);
@@ -665,11 +668,11 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
     const size_t plane_off = static_cast<size_t>(live ? plane : 0) * plane_elems;
     int l0 = 2;
-    if (pl.prefetch) {
+    if constexpr (MODE == 0) {
       if (live)
         plane_commit<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
                                    lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, ltid, sg);
-    } else if (pl.vec_ok) {
+    } else if constexpr (MODE == 1) {
       if (live)
         load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
                           lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, ltid, sg);
@@ -679,7 +682,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     }
     WT_LDS_BARRIER();
     WT_TICK(1);
-    if (pl.prefetch && u + static_cast<int>(gridDim.x) < nunits) {
+    if (MODE == 0 && u + static_cast<int>(gridDim.x) < nunits) {
       int pn, cn;
       locate(u + gridDim.x, pn, cn);
       if (pn >= 0) plane_fetch<T, kFetchPasses>(x + pn * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
