@@ -143,6 +143,7 @@ static int run_plane2d_mode(const void* x, void* out, const float* fw, const flo
 template <typename T, int K, int TJ1>
 static int run_plane2d(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
                        hipStream_t stream) {
+  if (pl.prefetch && pl.fuse >= 2) return run_plane2d_mode<T, K, TJ1, 3>(x, out, fw, fb, pl, stream);
   if (pl.prefetch) return run_plane2d_mode<T, K, TJ1, 0>(x, out, fw, fb, pl, stream);
   if (pl.vec_ok) return run_plane2d_mode<T, K, TJ1, 1>(x, out, fw, fb, pl, stream);
   return run_plane2d_mode<T, K, TJ1, 2>(x, out, fw, fb, pl, stream);

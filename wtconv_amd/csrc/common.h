@@ -24,6 +24,7 @@
 #define WT_CHUNK_FENCE() do {} while (0)
 #define WT_LAUNDER_UNIFORM_PTR(p) do {} while (0)
 #define WT_LAUNDER_LANE_INT(v) do {} while (0)
+#define WT_WAVE_PRIORITY(n) do {} while (0)
 typedef const float* wt_uniform_ptr;
 #else
 // Folded weights are read-only for the whole launch and indexed uniformly: the constant
@@ -61,6 +62,11 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 // are recomputed per iteration (a few integer ops) instead of being hoisted out of the loop
 // into long-lived registers that end up spilled.
 #define WT_LAUNDER_LANE_INT(v) asm volatile("" : "+v"(v))
+// Issue priority of this wave against the other waves of its SIMD (0 = default, 3 = highest).
+// The short serial phases of a plane (few work items, barrier after barrier) run at high
+// priority so that they are not slowed down to a quarter of their speed by the arithmetic-heavy
+// phases of the other workgroups on the same SIMD, which fill whatever issue slots are left.
+#define WT_WAVE_PRIORITY(n) __builtin_amdgcn_s_setprio(n)
 #endif
 
 // Optional profiling aid (off in the product build): -DWT_PHASE_TIMING makes wave 0 of

@@ -613,8 +613,9 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 // the planes of one wave are the same channel of consecutive batch items, so the folded
 // weights stay wave-uniform (SGPRs).  The zero halos written once stay valid for every plane
 // (only interiors are rewritten).
-// MODE selects the loader at compile time (0: register prefetch of the next plane, 1: fused
-// vector load without prefetch, 2: element-wise load), so that the hot variant does not carry
+// MODE selects the loader at compile time (0: register prefetch of the next plane, 3: the same
+// with levels 2-3 produced at the commit, 1: fused vector load without prefetch, 2: element-wise
+// load), so that the hot variant does not carry
 // the registers of the others.
 template <typename T, int K, int TJ1, int TJC, int MODE>
 __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
@@ -649,13 +650,14 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     }
   };
 
+  constexpr bool kPrefetch = MODE == 0 || MODE == 3;
   WT_TICK_INIT();
   zero_lds(lds_all, pl.lds_floats);
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
   {
     int p0, c0;
     locate(blockIdx.x, p0, c0);
-    if (MODE == 0 && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
+    if (kPrefetch && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
   }
   WT_LDS_BARRIER();
   WT_TICK(0);
@@ -668,10 +670,19 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
     const size_t plane_off = static_cast<size_t>(live ? plane : 0) * plane_elems;
     int l0 = 2;
+    WT_WAVE_PRIORITY(3);
     if constexpr (MODE == 0) {
       if (live)
         plane_commit<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
                                    lds + pl.aoff[1], pl.astr[1], pl.apl[1], pl.P, ltid, sg);
+    } else if constexpr (MODE == 3) {   // one plane per workgroup: `live` is uniform
+      if (live) {
+        plane_commit_fused<kFetchPasses>(fa, fbuf, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P, lds + pl.aoff[1],
+                                         pl.astr[1], pl.apl[1], lds + pl.aoff[2], pl.astr[2], pl.apl[2],
+                                         lds + pl.aoff[pl.fuse], pl.astr[pl.fuse], pl.apl[pl.fuse], pl.P, pl.fuse,
+                                         ltid, sg);
+        l0 = pl.fuse + 1;
+      }
     } else if constexpr (MODE == 1) {
       if (live)
         load_analysis1<T>(x + plane_off, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], pl.P,
@@ -682,7 +693,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     }
     WT_LDS_BARRIER();
     WT_TICK(1);
-    if (MODE == 0 && u + static_cast<int>(gridDim.x) < nunits) {
+    if (kPrefetch && u + static_cast<int>(gridDim.x) < nunits) {
       int pn, cn;
       locate(u + gridDim.x, pn, cn);
       if (pn >= 0) plane_fetch<T, kFetchPasses>(x + pn * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
@@ -702,6 +713,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
       WT_TICK(1 + l);
     }
     WT_WAIT_VMEM();     // next plane's loads have landed; the stores below are not waited for
+    WT_WAVE_PRIORITY(0);
     if (live) synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off, ltid, sg);
     WT_LDS_BARRIER();   // the next plane overwrites the buffers read above
     WT_TICK(7);
@@ -885,6 +897,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     const bool valid = has_slot && b0 + slot < b_end;
     const size_t plane_off = (static_cast<size_t>(valid ? b0 + slot : b0) * pl.C + c) * plane_elems;
     int l0 = 2;
+    WT_WAVE_PRIORITY(3);
     if (pl.prefetch && pl.fuse >= 2) {      // one plane per iteration: every lane takes part
       plane_commit_fused<1>(xa, xb, pl.H, pl.W, lds + pl.aoff[0], pl.astr[0], P, lds + pl.aoff[1], pl.astr[1],
                             pl.apl[1], lds + pl.aoff[2], pl.astr[2], pl.apl[2], lds + pl.aoff[pl.fuse],
@@ -933,6 +946,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       WT_LDS_BARRIER();
     }
     WT_TICK(9);
+    WT_WAVE_PRIORITY(0);
     // Both roles run the same code on different planes (one code path keeps a single
     // register set for the sums).
     {

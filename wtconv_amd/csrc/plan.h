@@ -99,8 +99,7 @@ inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
     const int gs = pow2_ceil(pl->W / 4);       // 2x4 pieces per row pair, one lane each
     const int rows_per_pass = sg / gs;
     pl->prefetch = rows_per_pass >= 1 && (pl->h[1] + rows_per_pass - 1) / rows_per_pass <= kFetchPasses;
-    (void)gs;   // (measured: the fused commit does not pay in the plane kernel; it stays on in the
-                //  weight-gradient kernel, which builds two pyramids per plane)
+    if (pl->prefetch && sg == pl->block && gs <= 16 && pl->L >= 2) pl->fuse = pl->L >= 3 ? 3 : 2;
   }
 }
 
