@@ -124,10 +124,15 @@ def test_config4_1d_small_batch(hip_device):
 @pytest.mark.parametrize("shape,K,L,bias,stride", [
     ((2, 3, 37), 5, 3, True, 1),
     ((1, 2, 9), 3, 4, False, 1),
-    ((2, 2, 2500), 5, 4, True, 1),     # ragged last tile
-    ((1, 3, 1000), 7, 5, True, 1),
+    ((2, 2, 2500), 5, 4, True, 1),     # row-resident kernels, ragged last lane
+    ((1, 3, 1000), 7, 5, True, 1),     # row-resident, level-5 edges from three lanes away
     ((2, 2, 51), 3, 2, True, 2),       # stride = true average pool
     ((1, 1, 1), 3, 1, True, 1),
+    ((3, 2, 517), 5, 3, True, 1),      # row-resident, 16 samples per lane, rows not 16-byte sized
+    ((2, 3, 700), 7, 3, False, 1),     # row-resident, K = 7
+    ((1, 2, 8192), 3, 2, True, 1),     # row-resident at the 512-lane limit
+    ((1, 2, 20000), 5, 4, True, 1),    # beyond it: tiled kernels, 20 tiles
+    ((5, 4, 4096), 5, 4, True, 1),     # several rows per chunk in the parameter-gradient kernel
 ])
 def test_edge_shapes_1d(hip_device, shape, K, L, bias, stride):
     _run_fp32("1d", shape[1], K, L, shape, hip_device, bias=bias, stride=stride, seed=5)

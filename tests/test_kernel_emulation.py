@@ -107,11 +107,24 @@ def _case1d(B, C, N, K, L, bias, seed=0):
     (2, 2, 64, 5, 3, True),
     (1, 2, 37, 5, 3, True),        # odd lengths at several levels
     (1, 1, 9, 3, 4, False),        # row shorter than 2^L
-    (1, 1, 2500, 5, 4, True),      # three tiles, ragged last tile
+    (1, 1, 2500, 5, 4, True),      # row-resident kernels: 79 lanes of 32 samples, ragged last lane
     (1, 2, 100, 7, 2, True),
     (1, 1, 40, 1, 2, True),
+    (2, 2, 1024, 5, 4, True),      # row-resident, exactly 32 full lanes, two rows per chunk
+    (1, 2, 517, 5, 3, True),       # row-resident, 16 samples per lane, odd length, scalar HBM path
+    (1, 1, 700, 7, 3, False),      # row-resident, K = 7: level 3 holds 2 < R entries per lane
+    (1, 1, 600, 3, 5, True),       # row-resident, five levels
+    (1, 1, 800, 5, 5, True),       # row-resident, one level-5 entry per lane: edges from two lanes away
+    (1, 1, 20000, 5, 4, True),     # longer than 512 lanes: tiled kernels, 20 tiles
 ])
 def test_emulated_1d_fp32(B, C, N, K, L, bias):
     x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, bias)
     got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K)
     _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
+
+
+def test_emulated_1d_row_resident_bf16():
+    x, g, bw, bb, bs, ws, ss = _case1d(2, 2, 1000, 5, 4, True)
+    x, g = _bf16_round(x), _bf16_round(g)
+    got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, 5, dtype=1)
+    _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=1e-2, atol_scale=1e-2)

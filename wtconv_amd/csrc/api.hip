@@ -6,6 +6,7 @@
 
 #include "common.h"
 #include "kernels1d.h"
+#include "kernels1d_row.h"
 #include "kernels2d.h"
 #include "plan.h"
 
@@ -297,6 +298,111 @@ static int run_wgrad1d_k(int K, int L, const void* x, const void* g, float* part
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
 
+// ---- row-resident 1-D kernels ----------------------------------------------------------
+// Rows of 16 to 512 lanes' worth of samples run on the register-resident kernels; shorter or
+// longer rows, K = 1 and (K, L) pairs whose lane would hold more than 32 samples use the tiled ones.
+static bool row1d_lanes(int N, int K, int L, int* nl, int* block) {
+  if (K < 3 || K > 7 || L < 1 || L > kMaxLevels) return false;
+  const int S = row1d_samples(K, L);
+  if (S > kRow1dMaxSamples) return false;
+  const int n = (N + S - 1) / S;
+  if (n < 16 || n > kRow1dMaxLanes) return false;
+  *nl = n;
+  *block = (n + 63) / 64 * 64;
+  return true;
+}
+
+static Row1D make_row1d(int C, int N, int nl, size_t esz, const void* p0, const void* p1) {
+  Row1D r = {};
+  r.C = C; r.N = N; r.nl = nl;
+  auto aligned = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  r.vec_ok = (static_cast<size_t>(N) * esz % 16 == 0) && aligned(p0) && aligned(p1);
+  return r;
+}
+
+// Rows per workgroup of the row-resident weight-gradient kernel: enough chunks to fill 256 CUs
+// at 8 waves each (a constant, so that workspace sizes do not depend on the device queried).
+static void row1d_chunks(int B, int C, int K, int L, int block, int* per_chunk, int* nchunk) {
+  const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
+  int per_cu = static_cast<int>(kLdsLimitBytes / lds);
+  if (per_cu > 512 / block) per_cu = 512 / block;
+  if (per_cu < 1) per_cu = 1;
+  int want = (256 * per_cu + C - 1) / C;
+  if (want < 1) want = 1;
+  if (want > B) want = B;
+  const int pc = (B + want - 1) / want;
+  *per_chunk = pc;
+  *nchunk = (B + pc - 1) / pc;
+}
+
+template <typename T, int K, int L>
+static int run_row1d(const void* x, void* out, const float* fw, const float* fb, const Row1D& pl, int B, int block,
+                     hipStream_t stream) {
+  if constexpr (row1d_built(K, L)) {
+    auto kern = wt1d_row_kernel<T, K, L>;
+    const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
+    if (int e = allow_lds(kern, lds)) return e;
+    const long long nrows = static_cast<long long>(B) * pl.C;
+    if (nrows > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "batch*channels = %lld is too large", nrows);
+    long long grid = static_cast<long long>(compute_units()) * resident_per_cu(kern, block, lds);
+    if (grid > nrows) grid = nrows;
+    WT_LAUNCH(kern, dim3(static_cast<unsigned>(grid)), dim3(block), lds, stream, static_cast<const T*>(x),
+              static_cast<T*>(out), fw, fb, pl, static_cast<int>(nrows));
+    return check_launch("wt1d_row_kernel");
+  } else {
+    return fail(WTCONV_E_UNSUPPORTED, "row-resident 1-D kernel not built for kernel_size %d, %d levels", K, L);
+  }
+}
+
+template <typename T, int K, int L>
+static int run_row1d_wgrad(const void* x, const void* g, float* partial, const Row1D& pl, int B, int block,
+                           int per_chunk, int nchunk, hipStream_t stream) {
+  if constexpr (row1d_built(K, L)) {
+    auto kern = wt1d_row_wgrad_kernel<T, K, L>;
+    const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
+    if (int e = allow_lds(kern, lds)) return e;
+    WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(block), lds, stream, static_cast<const T*>(x),
+              static_cast<const T*>(g), partial, pl, B, per_chunk);
+    return check_launch("wt1d_row_wgrad_kernel");
+  } else {
+    return fail(WTCONV_E_UNSUPPORTED, "row-resident 1-D kernel not built for kernel_size %d, %d levels", K, L);
+  }
+}
+
+#define WT_ROW1D_SWITCH_L(T, K, CALL)                                 \
+  switch (L) {                                                        \
+    case 1: return CALL(T, K, 1);                                     \
+    case 2: return CALL(T, K, 2);                                     \
+    case 3: return CALL(T, K, 3);                                     \
+    case 4: return CALL(T, K, 4);                                     \
+    case 5: return CALL(T, K, 5);                                     \
+  }                                                                   \
+  break;
+#define WT_ROW1D_SWITCH(T, CALL)                                      \
+  switch (K) {                                                        \
+    case 3: WT_ROW1D_SWITCH_L(T, 3, CALL)                             \
+    case 5: WT_ROW1D_SWITCH_L(T, 5, CALL)                             \
+    case 7: WT_ROW1D_SWITCH_L(T, 7, CALL)                             \
+  }
+
+template <typename T>
+static int run_row1d_kl(int K, int L, const void* x, void* out, const float* fw, const float* fb, const Row1D& pl,
+                        int B, int block, hipStream_t stream) {
+#define WT_CALL(T_, K_, L_) run_row1d<T_, K_, L_>(x, out, fw, fb, pl, B, block, stream)
+  WT_ROW1D_SWITCH(T, WT_CALL)
+#undef WT_CALL
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d / %d levels not built", K, L);
+}
+
+template <typename T>
+static int run_row1d_wgrad_kl(int K, int L, const void* x, const void* g, float* partial, const Row1D& pl, int B,
+                              int block, int per_chunk, int nchunk, hipStream_t stream) {
+#define WT_CALL(T_, K_, L_) run_row1d_wgrad<T_, K_, L_>(x, g, partial, pl, B, block, per_chunk, nchunk, stream)
+  WT_ROW1D_SWITCH(T, WT_CALL)
+#undef WT_CALL
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d / %d levels not built", K, L);
+}
+
 static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
                        int N, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes, void* stream_,
                        int flip) {
@@ -306,7 +412,9 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  if (static_cast<long long>(B) * C > 65535)
+  int nl = 0, block = 0;
+  const bool row_resident = row1d_lanes(N, K, L, &nl, &block);
+  if (!row_resident && static_cast<long long>(B) * C > 65535)
     return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld exceeds the grid limit 65535", fn,
                 static_cast<long long>(B) * C);
   const Plan1D pl = make_plan1d(C, N, K, L, false, esz, x, out, nullptr);
@@ -317,6 +425,11 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 2 * L) * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 2, L, K, flip, flip ? 0 : 1, stream)) return e;
+  if (row_resident) {
+    const Row1D rp = make_row1d(C, N, nl, esz, x, out);
+    return dtype == WTCONV_F32 ? run_row1d_kl<float>(K, L, x, out, fw, fb, rp, B, block, stream)
+                               : run_row1d_kl<bf16_t>(K, L, x, out, fw, fb, rp, B, block, stream);
+  }
   return dtype == WTCONV_F32 ? run_tile1d_k<float>(K, x, out, fw, fb, pl, B, stream)
                              : run_tile1d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
 }
@@ -427,8 +540,11 @@ size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     const Plan1D pl = make_plan1d(C, N, K, levels, true, 4, nullptr, nullptr, nullptr);
-    int per_chunk, nchunk;
-    wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
+    int per_chunk, nchunk, nl = 0, block = 0;
+    if (row1d_lanes(N, K, levels, &nl, &block))
+      row1d_chunks(B, C, K, levels, block, &per_chunk, &nchunk);
+    else
+      wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
     floats = static_cast<size_t>(nchunk) * C * ((1 + 2 * levels) * K + 1);
   } else {
     floats = fold_floats(C, 2, levels, K);
@@ -473,13 +589,25 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   if (workspace == nullptr || workspace_bytes < need)
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  int per_chunk, nchunk;
-  wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
+  int per_chunk, nchunk, nl = 0, block = 0;
+  const bool row_resident = row1d_lanes(N, K, L, &nl, &block);
+  if (row_resident)
+    row1d_chunks(B, C, K, L, block, &per_chunk, &nchunk);
+  else
+    wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
   if (nchunk > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
   float* partial = static_cast<float*>(workspace);
-  const int e = dtype == WTCONV_F32
-                    ? run_wgrad1d_k<float>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream)
-                    : run_wgrad1d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream);
+  int e;
+  if (row_resident) {
+    const Row1D rp = make_row1d(C, N, nl, esz, x, grad_out);
+    e = dtype == WTCONV_F32
+            ? run_row1d_wgrad_kl<float>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream)
+            : run_row1d_wgrad_kl<bf16_t>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream);
+  } else {
+    e = dtype == WTCONV_F32
+            ? run_wgrad1d_k<float>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream)
+            : run_wgrad1d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream);
+  }
   if (e) return e;
   GradTable gt = {};
   gt.base_weight = grads->base_weight;
