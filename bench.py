@@ -50,6 +50,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary dtype and per-kernel timing")
     ap.add_argument("--cpu-batch", type=int, default=16)
+    ap.add_argument("--only-1d", action="store_true",
+                    help="run only the WTConv1d(64,64,5,wt_levels=4) x[64,64,4096] workload and print its line")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain device copy of one activation tensor (calibrates rocprof's "
                          "FETCH_SIZE/WRITE_SIZE against a kernel of known traffic) and exit")
@@ -189,10 +191,48 @@ def bench_1d(torch, dev, steps, warmup):
         mod(x).backward(g)
 
     wall_ms, med_ms, _, _ = time_steps(torch, step, nsets, steps, warmup)
-    return {"workload": f"WTConv1d({C},{C},kernel_size={K},wt_levels={L}) fwd+bwd on x[{B},{C},{N}] fp32",
-            "ms_per_step": wall_ms, "sequences_per_s": B / (wall_ms * 1e-3),
-            "step_GBps": 5 * P * 4 / (wall_ms * 1e-3) / 1e9,
-            "step_frac_hbm": 5 * P * 4 / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    res = {"workload": f"WTConv1d({C},{C},kernel_size={K},wt_levels={L}) fwd+bwd on x[{B},{C},{N}] fp32",
+           "ms_per_step": wall_ms, "sequences_per_s": B / (wall_ms * 1e-3),
+           "step_GBps": 5 * P * 4 / (wall_ms * 1e-3) / 1e9,
+           "step_frac_hbm": 5 * P * 4 / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+    # per-entry-point timing through the C ABI (each call = parameter fold + one main kernel)
+    import ctypes
+    from wtconv_amd import _lib
+    from wtconv_amd import functional as Fn
+    lib = _lib.load()
+    pd, bw, bb, bs, ws, ss = Fn._prep_params(sets[0][0], mod.base_conv.weight, mod.base_conv.bias,
+                                             mod.base_scale.weight, [m.weight for m in mod.wavelet_convs],
+                                             [m.weight for m in mod.wavelet_scale])
+    tab = Fn._table(_lib.Params, bw, bb, bs, ws, ss)
+    f32 = lambda t: torch.empty(t.shape, dtype=torch.float32, device=dev)
+    gtab = Fn._table(_lib.ParamGrads, f32(bw), f32(bb), f32(bs), [f32(w) for w in ws], [f32(s_) for s_ in ss])
+    outs = [torch.empty_like(sets[i][0]) for i in range(nsets)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    wsz = max(lib.wtconv1d_workspace_bytes(B, C, N, K, L, p) for p in (0, 1, 2))
+    wsp = torch.empty(wsz, dtype=torch.uint8, device=dev)
+    P_ = Fn._ptr
+
+    def k_fwd(i):
+        assert lib.wtconv1d_forward(P_(sets[i][0]), P_(outs[i]), ctypes.byref(tab), B, C, N, K, L, 0, 0, P_(wsp),
+                                    wsz, stream) == 0, lib.wtconv_last_error()
+
+    def k_bwd_in(i):
+        assert lib.wtconv1d_backward_input(P_(sets[i][1]), P_(outs[i]), ctypes.byref(tab), B, C, N, K, L, 0, 0,
+                                           P_(wsp), wsz, stream) == 0, lib.wtconv_last_error()
+
+    def k_bwd_par(i):
+        assert lib.wtconv1d_backward_params(P_(sets[i][0]), P_(sets[i][1]), ctypes.byref(tab), ctypes.byref(gtab),
+                                            B, C, N, K, L, 0, 0, P_(wsp), wsz, stream) == 0, lib.wtconv_last_error()
+
+    kern = {}
+    for name, fn in (("wt1d_row_kernel(forward)", k_fwd), ("wt1d_row_kernel(backward_input)", k_bwd_in),
+                     ("wt1d_row_wgrad_kernel", k_bwd_par)):
+        _, med, mn, avg = time_steps(torch, fn, nsets, steps, warmup)
+        kern[name] = {"avg_ms": avg, "median_ms": med, "min_ms": mn, "algorithmic_bytes": 2 * P * 4,
+                      "GBps": 2 * P * 4 / (avg * 1e-3) / 1e9, "frac_hbm": 2 * P * 4 / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    res["kernels"] = kern
+    return res
 
 
 def bench_model(torch, dev, steps, warmup, batch=256):
@@ -269,6 +309,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": src.numel() * src.element_size(),
                           "bytes_written": src.numel() * src.element_size(), "launches": args.warmup + args.steps}))
+        return
+
+    if args.only_1d:
+        print(json.dumps(bench_1d(torch, dev, args.steps, args.warmup)))
         return
 
     main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup, per_kernel=True)

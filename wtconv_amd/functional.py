@@ -30,11 +30,19 @@ def _ptr(t):
 def _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss):
     """Contiguous parameter tensors in one dtype the kernels accept (fp32 or bf16)."""
     tensors = [base_w, base_s] + list(wt_ws) + list(wt_ss) + ([base_b] if base_b is not None else [])
-    dts = {t.dtype for t in tensors}
-    pd = dts.pop() if len(dts) == 1 else torch.float32
-    if pd not in _DT:
+    pd = base_w.dtype
+    if pd not in _DT or any(t.dtype != pd for t in tensors):
         pd = torch.float32
-    conv = lambda t: None if t is None else t.detach().to(device=x.device, dtype=pd).contiguous()
+    dev = x.device
+
+    def conv(t):
+        if t is None:
+            return None
+        t = t.detach()
+        if t.dtype != pd or t.device != dev:
+            t = t.to(device=dev, dtype=pd)
+        return t if t.is_contiguous() else t.contiguous()
+
     return pd, conv(base_w), conv(base_b), conv(base_s), [conv(w) for w in wt_ws], [conv(s) for s in wt_ss]
 
 
@@ -56,8 +64,37 @@ def _check_input(x, ndim, what):
         raise TypeError(f"{what} supports float32 and bfloat16 activations, got {x.dtype}")
 
 
-def _workspace(nbytes, device):
-    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+_WS_BYTES = {}
+
+
+def _workspace_bytes(lib, dims, shape, K, L, which):
+    """Workspace size of one pass (the library's answer depends on the sizes only: cached)."""
+    key = (dims, shape, K, L, which)
+    n = _WS_BYTES.get(key)
+    if n is None:
+        fn = lib.wtconv2d_workspace_bytes if dims == 2 else lib.wtconv1d_workspace_bytes
+        n = max(int(fn(*shape, K, L, which)), 256)
+        _WS_BYTES[key] = n
+    return n
+
+
+class _on_device:
+    """Makes x's device current for the launches, only if it is not already."""
+
+    def __init__(self, device):
+        self.idx = device.index if device.index is not None else torch.cuda.current_device()
+        self.prev = None
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 class _WTConvFn(torch.autograd.Function):
@@ -68,26 +105,22 @@ class _WTConvFn(torch.autograd.Function):
     def forward(ctx, x, base_w, base_b, base_s, dims, K, L, *wt):
         wt_ws, wt_ss = wt[:L], wt[L:]
         lib = _lib.load()
-        x = x.contiguous()
+        if not x.is_contiguous():
+            x = x.contiguous()
         pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
-        out = torch.empty_like(x)
-        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
-        stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
-        with torch.cuda.device(x.device):
-            if dims == 2:
-                B, C, H, W = x.shape
-                wsz = lib.wtconv2d_workspace_bytes(B, C, H, W, K, L, _lib.PASS_FORWARD)
-                wsp = _workspace(wsz, x.device)
-                rc = lib.wtconv2d_forward(_ptr(x), _ptr(out), ctypes.byref(tab), B, C, H, W, K, L,
-                                          _DT[x.dtype], _DT[pd], _ptr(wsp), wsp.numel(), stream)
-            else:
-                B, C, N = x.shape
-                wsz = lib.wtconv1d_workspace_bytes(B, C, N, K, L, _lib.PASS_FORWARD)
-                wsp = _workspace(wsz, x.device)
-                rc = lib.wtconv1d_forward(_ptr(x), _ptr(out), ctypes.byref(tab), B, C, N, K, L,
-                                          _DT[x.dtype], _DT[pd], _ptr(wsp), wsp.numel(), stream)
-        _lib.check(rc, "wtconv forward")
-        ctx.dims, ctx.K, ctx.L, ctx.has_bias = dims, K, L, base_b is not None
+        shape = tuple(x.shape)
+        with _on_device(x.device):
+            out = torch.empty_like(x)
+            tab = _table(_lib.Params, bw, bb, bs, ws, ss)
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            wsz = _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_FORWARD)
+            wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
+            fn = lib.wtconv2d_forward if dims == 2 else lib.wtconv1d_forward
+            rc = fn(x.data_ptr(), out.data_ptr(), ctypes.byref(tab), *shape, K, L, _DT[x.dtype], _DT[pd],
+                    wsp.data_ptr(), wsz, stream)
+        if rc:
+            _lib.check(rc, "wtconv forward")
+        ctx.dims, ctx.K, ctx.L = dims, K, L
         ctx.save_for_backward(x, base_w, base_b, base_s, *wt)
         return out
 
@@ -97,54 +130,61 @@ class _WTConvFn(torch.autograd.Function):
         dims, K, L = ctx.dims, ctx.K, ctx.L
         wt_ws, wt_ss = wt[:L], wt[L:]
         lib = _lib.load()
-        g = grad_out.to(x.dtype).contiguous()
+        g = grad_out
+        if g.dtype != x.dtype:
+            g = g.to(x.dtype)
+        if not g.is_contiguous():
+            g = g.contiguous()
         pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
-        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
-        stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
         shape = tuple(x.shape)
         grad_x = None
         grads = [None] * (3 + 2 * L)
+        need_x = ctx.needs_input_grad[0]
         need_params = any(ctx.needs_input_grad[i] for i in (1, 2, 3)) or any(ctx.needs_input_grad[7:])
-        with torch.cuda.device(x.device):
-            if ctx.needs_input_grad[0]:
+        with _on_device(x.device):
+            tab = _table(_lib.Params, bw, bb, bs, ws, ss)
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            # one workspace for both passes: they run back to back on one stream
+            wsz = max(_workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_INPUT) if need_x else 0,
+                      _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_PARAMS) if need_params else 0,
+                      256)
+            wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
+            dt, pdt = _DT[x.dtype], _DT[pd]
+            if need_x:
                 grad_x = torch.empty_like(x)
-                if dims == 2:
-                    wsz = lib.wtconv2d_workspace_bytes(*shape, K, L, _lib.PASS_BACKWARD_INPUT)
-                    wsp = _workspace(wsz, x.device)
-                    rc = lib.wtconv2d_backward_input(_ptr(g), _ptr(grad_x), ctypes.byref(tab), *shape, K, L,
-                                                     _DT[x.dtype], _DT[pd], _ptr(wsp), wsp.numel(), stream)
-                else:
-                    wsz = lib.wtconv1d_workspace_bytes(*shape, K, L, _lib.PASS_BACKWARD_INPUT)
-                    wsp = _workspace(wsz, x.device)
-                    rc = lib.wtconv1d_backward_input(_ptr(g), _ptr(grad_x), ctypes.byref(tab), *shape, K, L,
-                                                     _DT[x.dtype], _DT[pd], _ptr(wsp), wsp.numel(), stream)
-                _lib.check(rc, "wtconv backward_input")
+                fn = lib.wtconv2d_backward_input if dims == 2 else lib.wtconv1d_backward_input
+                rc = fn(g.data_ptr(), grad_x.data_ptr(), ctypes.byref(tab), *shape, K, L, dt, pdt,
+                        wsp.data_ptr(), wsz, stream)
+                if rc:
+                    _lib.check(rc, "wtconv backward_input")
             if need_params:
-                f32 = lambda t: torch.empty(t.shape, dtype=torch.float32, device=x.device)
-                gbw, gbs = f32(bw), f32(bs)
-                gbb = f32(bb) if bb is not None else None
-                gws, gss = [f32(w) for w in ws], [f32(s) for s in ss]
-                gtab = _table(_lib.ParamGrads, gbw, gbb, gbs, gws, gss)
-                if dims == 2:
-                    wsz = lib.wtconv2d_workspace_bytes(*shape, K, L, _lib.PASS_BACKWARD_PARAMS)
-                    wsp = _workspace(wsz, x.device)
-                    rc = lib.wtconv2d_backward_params(_ptr(x), _ptr(g), ctypes.byref(tab), ctypes.byref(gtab),
-                                                      *shape, K, L, _DT[x.dtype], _DT[pd], _ptr(wsp),
-                                                      wsp.numel(), stream)
+                # one flat fp32 buffer for every gradient: a single allocation and, for bf16
+                # parameters, a single cast afterwards
+                plist = [bw, bs] + ([bb] if bb is not None else []) + list(ws) + list(ss)
+                sizes = [t.numel() for t in plist]
+                flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
+                views = flat.split(sizes)
+                nb = 3 if bb is not None else 2
+                gtab = _table(_lib.ParamGrads, views[0], views[2] if bb is not None else None, views[1],
+                              views[nb:nb + L], views[nb + L:])
+                fn = lib.wtconv2d_backward_params if dims == 2 else lib.wtconv1d_backward_params
+                rc = fn(x.data_ptr(), g.data_ptr(), ctypes.byref(tab), ctypes.byref(gtab), *shape, K, L, dt, pdt,
+                        wsp.data_ptr(), wsz, stream)
+                if rc:
+                    _lib.check(rc, "wtconv backward_params")
+                tensors = [base_w, base_s] + ([base_b] if base_b is not None else []) + list(wt_ws) + list(wt_ss)
+                out_dt = base_w.dtype
+                if all(t.dtype == out_dt for t in tensors):
+                    cast = flat.to(out_dt).split(sizes) if out_dt != torch.float32 else views
+                    outg = [v.view(t.shape) for v, t in zip(cast, tensors)]
                 else:
-                    wsz = lib.wtconv1d_workspace_bytes(*shape, K, L, _lib.PASS_BACKWARD_PARAMS)
-                    wsp = _workspace(wsz, x.device)
-                    rc = lib.wtconv1d_backward_params(_ptr(x), _ptr(g), ctypes.byref(tab), ctypes.byref(gtab),
-                                                      *shape, K, L, _DT[x.dtype], _DT[pd], _ptr(wsp),
-                                                      wsp.numel(), stream)
-                _lib.check(rc, "wtconv backward_params")
-                like = lambda gt, p: None if gt is None else gt.to(p.dtype).reshape(p.shape)
-                grads[0] = like(gbw, base_w)
-                grads[1] = like(gbb, base_b) if base_b is not None else None
-                grads[2] = like(gbs, base_s)
+                    outg = [v.to(t.dtype).view(t.shape) for v, t in zip(views, tensors)]
+                grads[0], grads[2] = outg[0], outg[1]
+                if base_b is not None:
+                    grads[1] = outg[2]
                 for i in range(L):
-                    grads[3 + i] = like(gws[i], wt_ws[i])
-                    grads[3 + L + i] = like(gss[i], wt_ss[i])
+                    grads[3 + i] = outg[nb + i]
+                    grads[3 + L + i] = outg[nb + L + i]
         return (grad_x, grads[0], grads[1], grads[2], None, None, None, *grads[3:])
 
 
