@@ -219,7 +219,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
   Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
   int tj1 = 4, sg_shift = 8;
-  choose_plane_shape(pl.h[1], pl.w[1], &tj1, &sg_shift);
+  choose_plane_shape(pl.h[1], pl.w[1], static_cast<size_t>(pl.plane_lds_floats) * 4, &tj1, &sg_shift);
   // keep the slots of a workgroup within LDS: fewer, larger plane groups if needed
   while (sg_shift < 8 && static_cast<size_t>(pl.plane_lds_floats) * 4 * (256 >> sg_shift) > kLdsLimitBytes / 2) ++sg_shift;
   finish_plane_plan(&pl, sg_shift);
