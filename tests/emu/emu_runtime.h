@@ -21,6 +21,9 @@
 #define __forceinline__ inline
 #define __launch_bounds__(...)
 #define __align__(n)
+// workgroups run one after the other here: a function-local static is shared by exactly the
+// threads of the running workgroup
+#define __shared__ static
 
 struct dim3 {
   unsigned x, y, z;

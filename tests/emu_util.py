@@ -12,7 +12,7 @@ BUILD_DIR = os.path.join(EMU_DIR, "_build")
 EXE = os.path.join(BUILD_DIR, "emu_driver")
 SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(EMU_DIR, "emu_driver.cpp")]
 DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
-                  ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "plan.h")] + [
+                  ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_stream.h", "plan.h")] + [
     os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
 
 

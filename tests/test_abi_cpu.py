@@ -40,6 +40,10 @@ def test_workspace_sizes(lib):
     assert par >= 4 * C * ((1 + 4 * L) * K * K + 1)
     assert lib.wtconv1d_workspace_bytes(64, 64, 4096, 5, 4, 0) >= 4 * (64 * 9 * 5 + 64)
     assert lib.wtconv2d_workspace_bytes(0, C, 56, 56, K, L, 0) == 0
+    # planes whose pyramid exceeds LDS: the workspace also holds the fp32 pyramid(s)
+    big = lib.wtconv2d_workspace_bytes(2, 4, 400, 400, K, L, 0)
+    assert big >= 4 * 2 * 4 * (400 * 400 + 200 * 200 * 4 // 4)
+    assert lib.wtconv2d_workspace_bytes(2, 4, 400, 400, K, L, 2) >= 2 * (big - fwd)
 
 
 def _params(L=2):
@@ -61,7 +65,7 @@ def _params(L=2):
     (dict(H=0), -1, "spatial size"),
     (dict(dtype=7), -1, "dtype"),
     (dict(x=0), -1, "null"),
-    (dict(H=400, W=400), -2, "too large"),
+    (dict(H=400, W=400), -3, "workspace"),     # larger than LDS: the HBM pyramid needs a larger workspace
     (dict(ws_bytes=16), -3, "workspace"),
 ])
 def test_forward_argument_validation(lib, kw, code, needle):
@@ -93,7 +97,7 @@ def test_check_raises_python_exceptions(lib):
     with pytest.raises(ValueError, match="odd and positive"):
         _lib.check(rc, "forward")
     rc = lib.wtconv2d_forward(0x1000, 0x2000, ctypes.byref(p), 2, 4, 400, 400, 5, 2, 0, 0, 0x3000, 1 << 20, None)
-    with pytest.raises(RuntimeError, match="too large"):
+    with pytest.raises(RuntimeError, match="workspace of"):
         _lib.check(rc, "forward")
 
 

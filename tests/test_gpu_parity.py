@@ -63,6 +63,10 @@ def test_stage_shapes_fp32_small_batch(hip_device, C, H, L):
     ((2, 2, 56, 56), 5, 5, True),      # model stage 1: 56 28 14 7 4 2
     ((1, 1, 1, 1), 3, 1, True),        # smallest plane
     ((2, 3, 33, 17), 5, 4, True),
+    ((2, 3, 160, 150), 5, 3, True),    # pyramid larger than LDS: level-by-level kernels
+    ((1, 2, 131, 137), 7, 4, False),   # the same with odd sizes at every level, K = 7
+    ((2, 2, 200, 200), 3, 5, True),    # five levels on a large plane
+    ((2, 4, 100, 100), 5, 2, True),    # plane-resident forward, level-by-level weight gradients
 ])
 def test_edge_shapes_fp32(hip_device, shape, K, L, bias):
     _run_fp32("2d", shape[1], K, L, shape, hip_device, bias=bias, seed=3)
@@ -115,6 +119,20 @@ def test_stage_shapes_bf16_small_batch(hip_device, C, H, L, bf16_params):
     U.compare_all(got, want, U.assert_bf16)
 
 
+def test_large_plane_bf16(hip_device):
+    """mmseg-sized plane (128x128, five levels) in bf16: the level-by-level kernels keep the
+    pyramid in fp32, so the bf16 bar applies to the rounding at the HBM boundary only."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 4, 5, 5, (2, 4, 128, 128))
+    U.randomize_scales(ref)
+    rb = lambda t: t.to(torch.bfloat16).float()
+    x, g = rb(x), rb(g)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 5)
+    got = U.hip_run(mod, x, g, hip_device, dtype=torch.bfloat16)
+    want = U.oracle_run(ref, x, g, torch.float32)
+    U.compare_all(got, want, U.assert_bf16)
+
+
 # ------------------------------------------------------------------ 1-D
 def test_config4_1d_small_batch(hip_device):
     """WTConv1d(64,64,5,wt_levels=4) on rows of 4096 at batch 4."""
@@ -148,6 +166,32 @@ def test_1d_bf16(hip_device):
     got = U.hip_run(mod, x, g, hip_device, dtype=torch.bfloat16)
     want = U.oracle_run(ref, x, g, torch.float32)
     U.compare_all(got, want, U.assert_bf16)
+
+
+def test_under_autocast_and_channels_last(hip_device):
+    """torch.autocast(bf16) around the layer and a channels_last input: the layer takes fp32
+    activations with fp32 parameters as they are (the reference's convs would run in bf16
+    there and its scale multiply promotes back to fp32, wtconv2d.py:89-97), so the result
+    equals the plain fp32 call; a channels_last input is made contiguous first."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 8, 5, 2, (2, 8, 20, 20))
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 2).to(hip_device)
+    xd = x.to(hip_device)
+    plain = mod(xd)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        xa = xd.clone().requires_grad_(True)
+        auto = mod(xa)
+        auto.backward(g.to(hip_device))
+    assert auto.dtype == torch.float32
+    assert torch.equal(auto, plain)
+    assert xa.grad is not None and xa.grad.dtype == torch.float32
+    cl = mod(xd.contiguous(memory_format=torch.channels_last))
+    assert torch.equal(cl, plain)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        half_in = mod(xd.bfloat16())          # bf16 activations, fp32 parameters
+    assert half_in.dtype == torch.bfloat16
+    U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
 
 
 # ------------------------------------------------------------------ full-size checks

@@ -75,6 +75,8 @@ def _built():
     (1, 1, 28, 28, 5, 5, True),     # five levels: 28 14 7 4 2 1
     (5, 3, 7, 7, 5, 2, True),       # several small planes per workgroup / per wave, ragged batch tail
     (3, 2, 14, 14, 3, 2, True),     # 16 threads per plane, stacked planes in the weight-gradient kernel
+    (1, 1, 132, 141, 5, 3, True),   # pyramid larger than LDS: level-by-level kernels, odd sizes at levels 1-3
+    (2, 2, 100, 100, 3, 2, False),  # plane-resident forward, level-by-level weight gradients (two pyramids)
 ])
 def test_emulated_2d_fp32(B, C, H, W, K, L, bias):
     x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias)

@@ -6,7 +6,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libwtconv_hip.so")
 SOURCES = [os.path.join(CSRC, "api.hip")]
-HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "plan.h")] + [
+HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_stream.h", "plan.h")] + [
     os.path.join(os.path.dirname(PKG_DIR), "include", "wtconv_hip.h")]
 
 # packed-FP32 code generation is switched off on purpose: every float op is a scalar VALU op

@@ -8,6 +8,7 @@
 #include "kernels1d.h"
 #include "kernels1d_row.h"
 #include "kernels2d.h"
+#include "kernels2d_stream.h"
 #include "plan.h"
 
 namespace wt {
@@ -208,6 +209,142 @@ static int run_wgrad2d_k(int K, int L, const void* x, const void* g, float* part
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
 
+// ---- planes that do not fit LDS: level-by-level kernels through an HBM pyramid ----------
+static bool plane_fits_lds(int B, int C, int H, int W, int K, int L) {
+  Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, 4, nullptr, nullptr, nullptr);
+  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= kLdsLimitBytes;
+}
+
+static bool wgrad_fits_lds(int B, int C, int H, int W, int K, int L) {
+  Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, 4, nullptr, nullptr, nullptr, 1);
+  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= kLdsLimitBytes;
+}
+
+static size_t round_up64(size_t v) { return (v + 63) / 64 * 64; }
+
+static Stream2D make_stream2d(int B, int C, int H, int W, int L) {
+  Stream2D s = {};
+  s.C = C; s.H = H; s.W = W; s.L = L;
+  s.nplanes = B * C;
+  s.h[0] = H; s.w[0] = W;
+  size_t off = 0;
+  for (int l = 1; l <= L; ++l) {
+    s.h[l] = (s.h[l - 1] + 1) / 2;
+    s.w[l] = (s.w[l - 1] + 1) / 2;
+    s.aoff[l] = off;
+    off += round_up64(static_cast<size_t>(s.nplanes) * 4 * s.h[l] * s.w[l]);
+  }
+  for (int l = 2; l <= L; ++l) {
+    s.zoff[l] = off;
+    off += round_up64(static_cast<size_t>(s.nplanes) * s.h[l - 1] * s.w[l - 1]);
+  }
+  s.floats = off;
+  return s;
+}
+
+// Batch chunks of the streamed weight-gradient kernels: about 2048 workgroups per launch of
+// the four sub-band filters of a level (a constant rule: workspace sizes do not depend on the device).
+static void stream_chunks(int B, int C, int* bchunk, int* nchunk) {
+  int want = (2048 + 4 * C - 1) / (4 * C);
+  if (want < 1) want = 1;
+  if (want > B) want = B;
+  const int bc = (B + want - 1) / want;
+  *bchunk = bc;
+  *nchunk = (B + bc - 1) / bc;
+}
+
+template <typename T>
+static int stream_analysis_chain(const T* src, float* pyr, const Stream2D& sp, hipStream_t stream) {
+  const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
+  for (int l = 1; l <= sp.L; ++l) {
+    const int n = sp.h[l] * sp.w[l];
+    const unsigned gx = static_cast<unsigned>((n + 255) / 256);
+    if (l == 1) {
+      WT_LAUNCH(stream_analysis_kernel<T>, dim3(gx, gy), dim3(256), 0, stream, src,
+                static_cast<size_t>(sp.H) * sp.W, sp.H, sp.W, pyr + sp.aoff[1], sp.h[1], sp.w[1], sp.nplanes);
+    } else {
+      WT_LAUNCH(stream_analysis_kernel<float>, dim3(gx, gy), dim3(256), 0, stream,
+                static_cast<const float*>(pyr + sp.aoff[l - 1]), static_cast<size_t>(4) * sp.h[l - 1] * sp.w[l - 1],
+                sp.h[l - 1], sp.w[l - 1], pyr + sp.aoff[l], sp.h[l], sp.w[l], sp.nplanes);
+    }
+    if (int e = check_launch("stream_analysis_kernel")) return e;
+  }
+  return 0;
+}
+
+template <typename T, int K>
+static int run_stream2d(const void* x_, void* out_, const float* fw, const float* fb, float* pyr, const Stream2D& sp,
+                        hipStream_t stream) {
+  const T* x = static_cast<const T*>(x_);
+  T* out = static_cast<T*>(out_);
+  if (int e = stream_analysis_chain<T>(x, pyr, sp, stream)) return e;
+  const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
+  const int NF = 1 + 4 * sp.L;
+  for (int l = sp.L; l >= 1; --l) {
+    const unsigned tiles = static_cast<unsigned>(((sp.h[l] + kStreamTile - 1) / kStreamTile) *
+                                                 ((sp.w[l] + kStreamTile - 1) / kStreamTile));
+    const float* zin = l < sp.L ? pyr + sp.zoff[l + 1] : nullptr;
+    if (l > 1) {
+      WT_LAUNCH((stream_synth_kernel<T, K, false>), dim3(tiles, gy), dim3(256), 0, stream,
+                static_cast<const float*>(pyr + sp.aoff[l]), sp.h[l], sp.w[l], zin, pyr + sp.zoff[l], sp.h[l - 1],
+                sp.w[l - 1], static_cast<const T*>(nullptr), static_cast<T*>(nullptr), fw, fb, sp.C, NF,
+                1 + 4 * (l - 1), sp.nplanes);
+    } else {
+      WT_LAUNCH((stream_synth_kernel<T, K, true>), dim3(tiles, gy), dim3(256), 0, stream,
+                static_cast<const float*>(pyr + sp.aoff[1]), sp.h[1], sp.w[1], zin, static_cast<float*>(nullptr), sp.H,
+                sp.W, x, out, fw, fb, sp.C, NF, 1, sp.nplanes);
+    }
+    if (int e = check_launch("stream_synth_kernel")) return e;
+  }
+  return 0;
+}
+
+template <typename T>
+static int run_stream2d_k(int K, const void* x, void* out, const float* fw, const float* fb, float* pyr,
+                          const Stream2D& sp, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_stream2d<T, 1>(x, out, fw, fb, pyr, sp, stream);
+    case 3: return run_stream2d<T, 3>(x, out, fw, fb, pyr, sp, stream);
+    case 5: return run_stream2d<T, 5>(x, out, fw, fb, pyr, sp, stream);
+    case 7: return run_stream2d<T, 7>(x, out, fw, fb, pyr, sp, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
+template <typename T, int K>
+static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, float* pyr_x, float* pyr_g,
+                              const Stream2D& sp, int B, int bchunk, int nchunk, hipStream_t stream) {
+  const T* x = static_cast<const T*>(x_);
+  const T* g = static_cast<const T*>(g_);
+  if (int e = stream_analysis_chain<T>(x, pyr_x, sp, stream)) return e;
+  if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream)) return e;
+  const int rec = (1 + 4 * sp.L) * K * K + 1;
+  WT_LAUNCH((stream_corr_kernel<T, K>), dim3(sp.C, nchunk), dim3(256), 0, stream, x, g,
+            static_cast<size_t>(sp.H) * sp.W, static_cast<size_t>(0), sp.H, sp.W, partial, rec, 0, 1, 1, B, sp.C,
+            bchunk);
+  if (int e = check_launch("stream_corr_kernel")) return e;
+  for (int l = 1; l <= sp.L; ++l) {
+    const size_t n = static_cast<size_t>(sp.h[l]) * sp.w[l];
+    WT_LAUNCH((stream_corr_kernel<float, K>), dim3(sp.C * 4, nchunk), dim3(256), 0, stream,
+              static_cast<const float*>(pyr_x + sp.aoff[l]), static_cast<const float*>(pyr_g + sp.aoff[l]), 4 * n, n,
+              sp.h[l], sp.w[l], partial, rec, 1 + 4 * (l - 1), 4, 0, B, sp.C, bchunk);
+    if (int e = check_launch("stream_corr_kernel")) return e;
+  }
+  return 0;
+}
+
+template <typename T>
+static int run_stream2d_wgrad_k(int K, const void* x, const void* g, float* partial, float* pyr_x, float* pyr_g,
+                                const Stream2D& sp, int B, int bchunk, int nchunk, hipStream_t stream) {
+  switch (K) {
+    case 1: return run_stream2d_wgrad<T, 1>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+    case 3: return run_stream2d_wgrad<T, 3>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+    case 5: return run_stream2d_wgrad<T, 5>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+    case 7: return run_stream2d_wgrad<T, 7>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+  }
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
+}
+
 static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
                         int H, int W, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes,
                         void* stream_, int flip) {
@@ -217,6 +354,21 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
+  if (ws == nullptr || ws_bytes < need)
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
+  if (static_cast<long long>(B) * C > 0x7fffffffLL / 4)
+    return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld is too large", fn, static_cast<long long>(B) * C);
+  if (!plane_fits_lds(B, C, H, W, K, L)) {
+    const Stream2D sp = make_stream2d(B, C, H, W, L);
+    float* fw = static_cast<float*>(ws);
+    float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
+    float* pyr = fw + round_up64(fold_floats(C, 4, L, K * K));
+    if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
+    return dtype == WTCONV_F32 ? run_stream2d_k<float>(K, x, out, fw, fb, pyr, sp, stream)
+                               : run_stream2d_k<bf16_t>(K, x, out, fw, fb, pyr, sp, stream);
+  }
   Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
   int tj1 = 4, sg_shift = 8;
   choose_plane_shape(pl.h[1], pl.w[1], static_cast<size_t>(pl.plane_lds_floats) * 4, &tj1, &sg_shift);
@@ -227,10 +379,6 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
     return fail(WTCONV_E_UNSUPPORTED,
                 "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
                 "plane-resident kernels", fn, H, W, L, static_cast<size_t>(pl.lds_floats) * 4, kLdsLimitBytes);
-  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
-  if (ws == nullptr || ws_bytes < need)
-    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
@@ -466,10 +614,17 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     int bchunk, nchunk;
-    wgrad_chunks(B, C, wgrad_planes_per_iter(B, H, W, K, levels), kWgradResident, &bchunk, &nchunk);
-    floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
+    if (wgrad_fits_lds(B, C, H, W, K, levels)) {
+      wgrad_chunks(B, C, wgrad_planes_per_iter(B, H, W, K, levels), kWgradResident, &bchunk, &nchunk);
+      floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
+    } else {      // partial sums, then the pyramids of x and of grad_out
+      stream_chunks(B, C, &bchunk, &nchunk);
+      floats = round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1)) +
+               2 * make_stream2d(B, C, H, W, levels).floats;
+    }
   } else {
     floats = fold_floats(C, 4, levels, K * K);
+    if (!plane_fits_lds(B, C, H, W, K, levels)) floats = round_up64(floats) + make_stream2d(B, C, H, W, levels).floats;
   }
   return (floats * sizeof(float) + 255) / 256 * 256;
 }
@@ -506,23 +661,32 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  const int pb = wgrad_planes_per_iter(B, H, W, K, L);
-  Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
-  finish_wgrad_plan(&pl);
-  if (static_cast<size_t>(pl.lds_floats) * 4 > kLdsLimitBytes)
-    return fail(WTCONV_E_UNSUPPORTED,
-                "%s: a %dx%d plane with %d levels needs %zu B of LDS (limit %d); plane too large for the "
-                "plane-resident kernels", fn, H, W, L, static_cast<size_t>(pl.lds_floats) * 4, kLdsLimitBytes);
   const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD_PARAMS);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+  if (static_cast<long long>(B) * C > 0x7fffffffLL / 4)
+    return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld is too large", fn, static_cast<long long>(B) * C);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   int bchunk, nchunk;
-  wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
   float* partial = static_cast<float*>(workspace);
-  const int e = dtype == WTCONV_F32
-                    ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
-                    : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
+  int e;
+  if (wgrad_fits_lds(B, C, H, W, K, L)) {
+    const int pb = wgrad_planes_per_iter(B, H, W, K, L);
+    Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
+    finish_wgrad_plan(&pl);
+    wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
+    e = dtype == WTCONV_F32 ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+                            : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
+  } else {
+    const Stream2D sp = make_stream2d(B, C, H, W, L);
+    stream_chunks(B, C, &bchunk, &nchunk);
+    if (nchunk > 65535 || C > 0x7fffffff / 4) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
+    float* pyr_x = partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * L) * K * K + 1));
+    float* pyr_g = pyr_x + sp.floats;
+    e = dtype == WTCONV_F32
+            ? run_stream2d_wgrad_k<float>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream)
+            : run_stream2d_wgrad_k<bf16_t>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+  }
   if (e) return e;
   GradTable gt = {};
   gt.base_weight = grads->base_weight;

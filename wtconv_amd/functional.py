@@ -101,7 +101,11 @@ class _WTConvFn(torch.autograd.Function):
     """dims = 2: x (B,C,H,W); dims = 1: x (B,C,N).  Argument order:
     x, base_w, base_b, base_s, dims, K, L, wt_w[0..L-1], wt_s[0..L-1]."""
 
+    # Under torch.autocast the inputs are taken as they come (fp32 or bf16 activations, fp32 or
+    # bf16 parameters, any mix): the kernels accumulate in fp32 either way, so there is nothing
+    # to down-cast; the decorators only make backward run with autocast off, as forward did.
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, x, base_w, base_b, base_s, dims, K, L, *wt):
         wt_ws, wt_ss = wt[:L], wt[L:]
         lib = _lib.load()
@@ -125,6 +129,7 @@ class _WTConvFn(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         x, base_w, base_b, base_s, *wt = ctx.saved_tensors
         dims, K, L = ctx.dims, ctx.K, ctx.L
