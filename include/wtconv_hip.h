@@ -33,7 +33,7 @@ enum { WTCONV_F32 = 0, WTCONV_BF16 = 1 };
 enum {
   WTCONV_OK = 0,
   WTCONV_E_ARG = -1,        /* bad shape / dtype / null pointer / alignment          */
-  WTCONV_E_UNSUPPORTED = -2,/* kernel size or plane too large for the built kernels  */
+  WTCONV_E_UNSUPPORTED = -2,/* kernel size or tensor extent beyond the built kernels    */
   WTCONV_E_WORKSPACE = -3,  /* workspace too small                                   */
   WTCONV_E_LAUNCH = -4      /* HIP reported a launch error                           */
 };
