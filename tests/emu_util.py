@@ -22,7 +22,8 @@ def build(force=False):
         newest = max(os.path.getmtime(p) for p in DEPS)
         if os.path.getmtime(EXE) >= newest:
             return EXE
-    cmd = ["g++", "-std=c++20", "-O1", "-g", "-fsanitize=address,undefined",
+    # -O0 -g1: the run time is dominated by thread creation, the build time by optimisation
+    cmd = ["g++", "-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined",
            "-fno-sanitize-recover=undefined", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
            SOURCES[0], SOURCES[1], "-pthread", "-o", EXE]
     subprocess.run(cmd, check=True, cwd=ROOT)
