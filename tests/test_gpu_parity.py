@@ -257,6 +257,63 @@ def test_config2_full_size_param_grads_vs_oracle(hip_device):
         print(f"\n{n}: max|hip-fp64| = {e_hip:.3e}, max|cpu_fp32-fp64| = {e_cpu:.3e}, max|want| = {want.abs().max():.1f}")
 
 
+
+def _full_size_properties(kind, C, K, L, shape, hip_device, dtype, nsample=2):
+    """Full-size run of one configuration: the first `nsample` batch items against the oracle
+    (planes / rows are independent), the adjoint identity <f(x) - bias response, g> = <x, f^T g>
+    over the whole batch (accumulated in float64 on the device) and additivity of the
+    parameter gradients over two half batches."""
+    W2, W1 = _mods()
+    ref, x, g = U.seeded_case(kind, C, K, L, shape)
+    U.randomize_scales(ref)
+    bf16 = dtype == torch.bfloat16
+    if bf16:
+        x, g = x.to(dtype).float(), g.to(dtype).float()
+    mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, K, L).to(hip_device)
+    xd = x.to(hip_device, dtype).requires_grad_(True)
+    gd = g.to(hip_device, dtype)
+    out = mod(xd)
+    out.backward(gd)
+    torch.cuda.synchronize()
+    check = U.assert_bf16 if bf16 else U.assert_fp32
+    wo, wdx, _ = U.oracle_run(ref, x[:nsample], g[:nsample], torch.float32 if bf16 else torch.float64)
+    check(out[:nsample].detach().float().cpu(), wo.float(), f"out[:{nsample}]")
+    check(xd.grad[:nsample].float().cpu(), wdx.float(), f"grad_x[:{nsample}]")
+    view = (1, -1, 1, 1) if kind == "2d" else (1, -1, 1)
+    bias_resp = (mod.base_scale.weight * mod.base_conv.bias.view(*view)).detach()
+    lhs = ((out.detach().double() - bias_resp.double()) * gd.double()).sum().item()
+    rhs = (xd.detach().double() * xd.grad.double()).sum().item()
+    # out and grad_x are each rounded once to the activation dtype: the two inner products
+    # then differ by a random walk of rounding errors, far below the bound used here
+    norm = (out.detach().double().norm() * gd.double().norm()).item()
+    tol = (4e-3 if bf16 else 1e-6) * norm / (out.numel() ** 0.5) * 10 + (1e-6 * abs(lhs))
+    assert abs(lhs - rhs) <= tol, (lhs, rhs, tol)
+    full = {n: p.grad.clone() for n, p in mod.named_parameters() if p.grad is not None}
+    B = shape[0]
+    acc = None
+    for sl in (slice(0, B // 2), slice(B // 2, B)):
+        for p in mod.parameters():
+            p.grad = None
+        xs = x[sl].to(hip_device, dtype).requires_grad_(True)
+        mod(xs).backward(g[sl].to(hip_device, dtype))
+        cur = {n: p.grad.clone() for n, p in mod.named_parameters() if p.grad is not None}
+        acc = cur if acc is None else {n: acc[n] + cur[n] for n in acc}
+    for n in full:
+        scale = full[n].abs().max().item()
+        assert (full[n] - acc[n]).abs().max().item() <= 2e-5 * scale + 1e-4, n
+
+
+@pytest.mark.parametrize("name,C,L,H", [("2b", 96, 3, 56), ("3a", 192, 3, 28), ("3b", 384, 2, 14), ("3c", 768, 2, 7)])
+def test_full_size_bf16_configs(hip_device, name, C, L, H):
+    """BASELINE configurations 2b / 3a / 3b / 3c at their full sizes (batch 128, bf16)."""
+    _full_size_properties("2d", C, 5, L, (128, C, H, H), hip_device, torch.bfloat16)
+
+
+def test_config4_full_size_1d(hip_device):
+    """WTConv1d(64,64,5,wt_levels=4) on x[64,64,4096] fp32 at full size."""
+    _full_size_properties("1d", 64, 5, 4, (64, 64, 4096), hip_device, torch.float32)
+
+
 # ------------------------------------------------------------------ caller harness
 def test_wtconvnext_harness_hip_vs_oracle_conv_class(hip_device):
     """WTConvNeXt-T (reduced depth) with the HIP WTConv2d against the same host model with the
