@@ -194,6 +194,31 @@ def test_under_autocast_and_channels_last(hip_device):
     U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
 
 
+def test_torch_compile_custom_op(hip_device):
+    """Under torch.compile the layer is an opaque torch.library operator with a fake
+    (shape-only) implementation and a registered backward: the compiled module traces as one
+    graph and gives the eager results, forward and every gradient."""
+    W2, W1 = _mods()
+    for kind, cls, shape in (("2d", W2, (2, 6, 20, 24)), ("1d", W1, (2, 6, 640))):
+        ref, x, g = U.seeded_case(kind, 6, 5, 2, shape)
+        U.randomize_scales(ref)
+        mod = U.copy_to_hip_module(ref, cls, kind, 5, 2).to(hip_device)
+        xe = x.to(hip_device).requires_grad_(True)
+        oe = mod(xe)
+        oe.backward(g.to(hip_device))
+        eager = {n: p.grad.clone() for n, p in mod.named_parameters() if p.grad is not None}
+        for p in mod.parameters():
+            p.grad = None
+        cmod = torch.compile(mod, backend="aot_eager", fullgraph=True)
+        xc = x.to(hip_device).requires_grad_(True)
+        oc = cmod(xc)
+        oc.backward(g.to(hip_device))
+        assert torch.equal(oc, oe) and torch.equal(xc.grad, xe.grad)
+        for n, p in mod.named_parameters():
+            if n in eager:
+                assert torch.equal(p.grad, eager[n]), n
+
+
 # ------------------------------------------------------------------ full-size checks
 def test_config2_full_size_fp32(hip_device):
     """WTConv2d(96,96,5,wt_levels=3) on x[128,96,56,56]: forward/input-gradient planes are

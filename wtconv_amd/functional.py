@@ -5,6 +5,7 @@ wavelet level, the inverse cascade); PyTorch only supplies device memory and the
 Semantics follow the reference layer (wtconv/wtconv2d.py:38-87, wtconv/wtconv1d.py:38-87).
 """
 import ctypes
+from typing import List, Optional
 
 import torch
 
@@ -18,6 +19,8 @@ def check_kernel_size(kernel_size):
     fast_wtconv/cuda_haar/haar_cuda.py:86-105)."""
     if not isinstance(kernel_size, int) or kernel_size < 1 or kernel_size % 2 == 0:
         raise ValueError(f"kernel_size must be odd and positive, got {kernel_size}")
+    if torch.compiler.is_compiling():     # no ctypes under tracing; modules check at construction
+        return
     kmax = _lib.load().wtconv_max_kernel_size()
     if kernel_size > kmax:
         raise ValueError(f"kernel_size {kernel_size} exceeds the largest built kernel ({kmax})")
@@ -97,6 +100,87 @@ class _on_device:
         return False
 
 
+def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
+    """One forward launch sequence; returns (out, contiguous x)."""
+    lib = _lib.load()
+    if not x.is_contiguous():
+        x = x.contiguous()
+    pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    shape = tuple(x.shape)
+    with _on_device(x.device):
+        out = torch.empty_like(x)
+        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        wsz = _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_FORWARD)
+        wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
+        fn = lib.wtconv2d_forward if dims == 2 else lib.wtconv1d_forward
+        rc = fn(x.data_ptr(), out.data_ptr(), ctypes.byref(tab), *shape, K, L, _DT[x.dtype], _DT[pd],
+                wsp.data_ptr(), wsz, stream)
+    if rc:
+        _lib.check(rc, "wtconv forward")
+    return out, x
+
+
+def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L, need_x, need_params):
+    """grad_x (or None) and the parameter gradients in the order base_w, base_b (or None),
+    base_s, wt_ws[0..L-1], wt_ss[0..L-1] (all None when not needed), in the parameters' dtypes."""
+    lib = _lib.load()
+    g = grad_out
+    if g.dtype != x.dtype:
+        g = g.to(x.dtype)
+    if not g.is_contiguous():
+        g = g.contiguous()
+    pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    shape = tuple(x.shape)
+    grad_x = None
+    grads = [None] * (3 + 2 * L)
+    with _on_device(x.device):
+        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        # one workspace for both passes: they run back to back on one stream
+        wsz = max(_workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_INPUT) if need_x else 0,
+                  _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_PARAMS) if need_params else 0,
+                  256)
+        wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
+        dt, pdt = _DT[x.dtype], _DT[pd]
+        if need_x:
+            grad_x = torch.empty_like(x)
+            fn = lib.wtconv2d_backward_input if dims == 2 else lib.wtconv1d_backward_input
+            rc = fn(g.data_ptr(), grad_x.data_ptr(), ctypes.byref(tab), *shape, K, L, dt, pdt,
+                    wsp.data_ptr(), wsz, stream)
+            if rc:
+                _lib.check(rc, "wtconv backward_input")
+        if need_params:
+            # one flat fp32 buffer for every gradient: a single allocation and, for bf16
+            # parameters, a single cast afterwards
+            plist = [bw, bs] + ([bb] if bb is not None else []) + list(ws) + list(ss)
+            sizes = [t.numel() for t in plist]
+            flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
+            views = flat.split(sizes)
+            nb = 3 if bb is not None else 2
+            gtab = _table(_lib.ParamGrads, views[0], views[2] if bb is not None else None, views[1],
+                          views[nb:nb + L], views[nb + L:])
+            fn = lib.wtconv2d_backward_params if dims == 2 else lib.wtconv1d_backward_params
+            rc = fn(x.data_ptr(), g.data_ptr(), ctypes.byref(tab), ctypes.byref(gtab), *shape, K, L, dt, pdt,
+                    wsp.data_ptr(), wsz, stream)
+            if rc:
+                _lib.check(rc, "wtconv backward_params")
+            tensors = [base_w, base_s] + ([base_b] if base_b is not None else []) + list(wt_ws) + list(wt_ss)
+            out_dt = base_w.dtype
+            if all(t.dtype == out_dt for t in tensors):
+                cast = flat.to(out_dt).split(sizes) if out_dt != torch.float32 else views
+                outg = [v.view(t.shape) for v, t in zip(cast, tensors)]
+            else:
+                outg = [v.to(t.dtype).view(t.shape) for v, t in zip(views, tensors)]
+            grads[0], grads[2] = outg[0], outg[1]
+            if base_b is not None:
+                grads[1] = outg[2]
+            for i in range(L):
+                grads[3 + i] = outg[nb + i]
+                grads[3 + L + i] = outg[nb + L + i]
+    return grad_x, grads
+
+
 class _WTConvFn(torch.autograd.Function):
     """dims = 2: x (B,C,H,W); dims = 1: x (B,C,N).  Argument order:
     x, base_w, base_b, base_s, dims, K, L, wt_w[0..L-1], wt_s[0..L-1]."""
@@ -107,23 +191,7 @@ class _WTConvFn(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, x, base_w, base_b, base_s, dims, K, L, *wt):
-        wt_ws, wt_ss = wt[:L], wt[L:]
-        lib = _lib.load()
-        if not x.is_contiguous():
-            x = x.contiguous()
-        pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
-        shape = tuple(x.shape)
-        with _on_device(x.device):
-            out = torch.empty_like(x)
-            tab = _table(_lib.Params, bw, bb, bs, ws, ss)
-            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            wsz = _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_FORWARD)
-            wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
-            fn = lib.wtconv2d_forward if dims == 2 else lib.wtconv1d_forward
-            rc = fn(x.data_ptr(), out.data_ptr(), ctypes.byref(tab), *shape, K, L, _DT[x.dtype], _DT[pd],
-                    wsp.data_ptr(), wsz, stream)
-        if rc:
-            _lib.check(rc, "wtconv forward")
+        out, x = _forward_impl(x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L)
         ctx.dims, ctx.K, ctx.L = dims, K, L
         ctx.save_for_backward(x, base_w, base_b, base_s, *wt)
         return out
@@ -133,64 +201,71 @@ class _WTConvFn(torch.autograd.Function):
     def backward(ctx, grad_out):
         x, base_w, base_b, base_s, *wt = ctx.saved_tensors
         dims, K, L = ctx.dims, ctx.K, ctx.L
-        wt_ws, wt_ss = wt[:L], wt[L:]
-        lib = _lib.load()
-        g = grad_out
-        if g.dtype != x.dtype:
-            g = g.to(x.dtype)
-        if not g.is_contiguous():
-            g = g.contiguous()
-        pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
-        shape = tuple(x.shape)
-        grad_x = None
-        grads = [None] * (3 + 2 * L)
-        need_x = ctx.needs_input_grad[0]
         need_params = any(ctx.needs_input_grad[i] for i in (1, 2, 3)) or any(ctx.needs_input_grad[7:])
-        with _on_device(x.device):
-            tab = _table(_lib.Params, bw, bb, bs, ws, ss)
-            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            # one workspace for both passes: they run back to back on one stream
-            wsz = max(_workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_INPUT) if need_x else 0,
-                      _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_PARAMS) if need_params else 0,
-                      256)
-            wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
-            dt, pdt = _DT[x.dtype], _DT[pd]
-            if need_x:
-                grad_x = torch.empty_like(x)
-                fn = lib.wtconv2d_backward_input if dims == 2 else lib.wtconv1d_backward_input
-                rc = fn(g.data_ptr(), grad_x.data_ptr(), ctypes.byref(tab), *shape, K, L, dt, pdt,
-                        wsp.data_ptr(), wsz, stream)
-                if rc:
-                    _lib.check(rc, "wtconv backward_input")
-            if need_params:
-                # one flat fp32 buffer for every gradient: a single allocation and, for bf16
-                # parameters, a single cast afterwards
-                plist = [bw, bs] + ([bb] if bb is not None else []) + list(ws) + list(ss)
-                sizes = [t.numel() for t in plist]
-                flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
-                views = flat.split(sizes)
-                nb = 3 if bb is not None else 2
-                gtab = _table(_lib.ParamGrads, views[0], views[2] if bb is not None else None, views[1],
-                              views[nb:nb + L], views[nb + L:])
-                fn = lib.wtconv2d_backward_params if dims == 2 else lib.wtconv1d_backward_params
-                rc = fn(x.data_ptr(), g.data_ptr(), ctypes.byref(tab), ctypes.byref(gtab), *shape, K, L, dt, pdt,
-                        wsp.data_ptr(), wsz, stream)
-                if rc:
-                    _lib.check(rc, "wtconv backward_params")
-                tensors = [base_w, base_s] + ([base_b] if base_b is not None else []) + list(wt_ws) + list(wt_ss)
-                out_dt = base_w.dtype
-                if all(t.dtype == out_dt for t in tensors):
-                    cast = flat.to(out_dt).split(sizes) if out_dt != torch.float32 else views
-                    outg = [v.view(t.shape) for v, t in zip(cast, tensors)]
-                else:
-                    outg = [v.to(t.dtype).view(t.shape) for v, t in zip(views, tensors)]
-                grads[0], grads[2] = outg[0], outg[1]
-                if base_b is not None:
-                    grads[1] = outg[2]
-                for i in range(L):
-                    grads[3 + i] = outg[nb + i]
-                    grads[3 + L + i] = outg[nb + L + i]
+        grad_x, grads = _backward_impl(grad_out, x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L,
+                                       ctx.needs_input_grad[0], need_params)
         return (grad_x, grads[0], grads[1], grads[2], None, None, None, *grads[3:])
+
+
+# ---------------------------------------------------------------------------------------------
+# The same two steps as opaque operators for torch.compile (train.py:629-632 of the reference
+# offers --torchcompile): Dynamo cannot trace through ctypes, so while compiling the layer is
+# routed through torch.library custom ops with shape-only fake implementations.
+@torch.library.custom_op("wtconv_amd::layer_forward", mutates_args=())
+def _op_forward(x: torch.Tensor, base_w: torch.Tensor, base_b: Optional[torch.Tensor], base_s: torch.Tensor,
+                wt_ws: List[torch.Tensor], wt_ss: List[torch.Tensor], dims: int) -> torch.Tensor:
+    out, _ = _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, int(base_w.shape[-1]), len(wt_ws))
+    return out
+
+
+@_op_forward.register_fake
+def _(x, base_w, base_b, base_s, wt_ws, wt_ss, dims):
+    return torch.empty_like(x, memory_format=torch.contiguous_format)
+
+
+@torch.library.custom_op("wtconv_amd::layer_backward", mutates_args=())
+def _op_backward(grad_out: torch.Tensor, x: torch.Tensor, base_w: torch.Tensor, base_b: Optional[torch.Tensor],
+                 base_s: torch.Tensor, wt_ws: List[torch.Tensor], wt_ss: List[torch.Tensor],
+                 dims: int) -> List[torch.Tensor]:
+    """[grad_x, grad_base_w, grad_base_s, grad_base_b (empty without bias), grads of wt_ws, grads of wt_ss]."""
+    L = len(wt_ws)
+    gx, gr = _backward_impl(grad_out, x.contiguous(), base_w, base_b, base_s, wt_ws, wt_ss, dims,
+                            int(base_w.shape[-1]), L, True, True)
+    # the eager path hands out views of one flat buffer; operator outputs may not alias
+    gb = gr[1].clone() if gr[1] is not None else x.new_empty(0)
+    return [gx, gr[0].clone(), gr[2].clone(), gb] + [t.clone() for t in gr[3:]]
+
+
+@_op_backward.register_fake
+def _(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims):
+    gb = torch.empty_like(base_b) if base_b is not None else x.new_empty(0)
+    return ([torch.empty_like(x, memory_format=torch.contiguous_format), torch.empty_like(base_w),
+             torch.empty_like(base_s), gb] + [torch.empty_like(t) for t in wt_ws] + [torch.empty_like(t) for t in wt_ss])
+
+
+def _op_setup_context(ctx, inputs, output):
+    x, base_w, base_b, base_s, wt_ws, wt_ss, dims = inputs
+    ctx.dims, ctx.L, ctx.has_bias = dims, len(wt_ws), base_b is not None
+    ctx.save_for_backward(x, base_w, base_s, *wt_ws, *wt_ss, *([base_b] if base_b is not None else []))
+
+
+def _op_autograd_backward(ctx, grad_out):
+    saved = ctx.saved_tensors
+    L = ctx.L
+    x, base_w, base_s = saved[:3]
+    wt_ws, wt_ss = list(saved[3:3 + L]), list(saved[3 + L:3 + 2 * L])
+    base_b = saved[3 + 2 * L] if ctx.has_bias else None
+    res = _op_backward(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, ctx.dims)
+    return (res[0], res[1], res[3] if ctx.has_bias else None, res[2], list(res[4:4 + L]), list(res[4 + L:]), None)
+
+
+_op_forward.register_autograd(_op_autograd_backward, setup_context=_op_setup_context)
+
+
+def _apply(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, dims, K, L):
+    if torch.compiler.is_compiling():
+        return _op_forward(x, base_weight, base_bias, base_scale, list(wt_weights), list(wt_scales), dims)
+    return _WTConvFn.apply(x, base_weight, base_bias, base_scale, dims, K, L, *wt_weights, *wt_scales)
 
 
 def _check_params(C, K, L, S, dims, base_w, base_b, base_s, wt_ws, wt_ss):
@@ -219,7 +294,7 @@ def wtconv2d(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, strid
         raise ValueError(f"wt_levels must be 1-{_lib.MAX_LEVELS}, got {L}")
     check_kernel_size(int(K))
     _check_params(C, K, L, 4, 2, base_weight, base_bias, base_scale, wt_weights, wt_scales)
-    out = _WTConvFn.apply(x, base_weight, base_bias, base_scale, 2, int(K), L, *wt_weights, *wt_scales)
+    out = _apply(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, 2, int(K), L)
     if stride > 1:
         out = out[:, :, ::stride, ::stride]
     return out
@@ -235,7 +310,7 @@ def wtconv1d(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, strid
         raise ValueError(f"wt_levels must be 1-{_lib.MAX_LEVELS}, got {L}")
     check_kernel_size(int(K))
     _check_params(C, K, L, 2, 1, base_weight, base_bias, base_scale, wt_weights, wt_scales)
-    out = _WTConvFn.apply(x, base_weight, base_bias, base_scale, 1, int(K), L, *wt_weights, *wt_scales)
+    out = _apply(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, 1, int(K), L)
     if stride > 1:
         out = torch.nn.functional.avg_pool1d(out, kernel_size=stride, stride=stride)
     return out
