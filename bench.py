@@ -172,7 +172,7 @@ def bench_layer(torch, dev, dtype_name, workload, steps, warmup, per_kernel=True
 
 
 def bench_1d(torch, dev, steps, warmup):
-    """BASELINE config 4: WTConv1d(64,64,5,wt_levels=4), fp32, fwd+bwd, x[64,64,4096]."""
+    """The 1-D benchmark configuration: WTConv1d(64,64,5,wt_levels=4), fp32, fwd+bwd, x[64,64,4096]."""
     from wtconv.wtconv1d import WTConv1d
     B, C, N, K, L = 64, 64, 4096, 5, 4
     P = B * C * N
@@ -236,7 +236,7 @@ def bench_1d(torch, dev, steps, warmup):
 
 
 def bench_model(torch, dev, steps, warmup, batch=256):
-    """BASELINE config 5: WTConvNeXt-T, random init (seed 0), bf16 inference on [batch,3,224,224]."""
+    """The whole-model benchmark configuration: WTConvNeXt-T, random init (seed 0), bf16 inference on [batch,3,224,224]."""
     import wtconvnext
     torch.manual_seed(0)
     model = wtconvnext.wtconvnext_tiny().to(dev).bfloat16().eval()

@@ -330,7 +330,7 @@ def _full_size_properties(kind, C, K, L, shape, hip_device, dtype, nsample=2):
 
 @pytest.mark.parametrize("name,C,L,H", [("2b", 96, 3, 56), ("3a", 192, 3, 28), ("3b", 384, 2, 14), ("3c", 768, 2, 7)])
 def test_full_size_bf16_configs(hip_device, name, C, L, H):
-    """BASELINE configurations 2b / 3a / 3b / 3c at their full sizes (batch 128, bf16)."""
+    """The bf16 benchmark configurations (stage 1-4 shapes of WTConvNeXt-T) at their full sizes (batch 128)."""
     _full_size_properties("2d", C, 5, L, (128, C, H, H), hip_device, torch.bfloat16)
 
 
@@ -373,7 +373,7 @@ def test_wtconvnext_harness_hip_vs_oracle_conv_class(hip_device):
 
 
 def test_wtconvnext_tiny_bf16_inference_runs(hip_device):
-    """The BASELINE config-5 model at a small batch: bf16 inference forward on the HIP layer,
+    """The whole-model benchmark configuration at a small batch: bf16 inference forward on the HIP layer,
     compared with the same bf16 model using the oracle conv class on the GPU (cuDNN-free
     torch ops), loose tolerance (bf16 end to end)."""
     import wtconvnext
