@@ -194,6 +194,15 @@ def test_under_autocast_and_channels_last(hip_device):
     U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
 
 
+def test_double_backward_raises(hip_device):
+    W2, _ = _mods()
+    mod = W2(4, 4, 3, wt_levels=1).to(hip_device)
+    x = torch.randn(1, 4, 8, 8, device=hip_device, requires_grad=True)
+    (gx,) = torch.autograd.grad(mod(x).sum(), x, create_graph=True)
+    with pytest.raises(RuntimeError, match="does not require grad|differentiable"):
+        gx.sum().backward()
+
+
 def test_torch_compile_custom_op(hip_device):
     """Under torch.compile the layer is an opaque torch.library operator with a fake
     (shape-only) implementation and a registered backward: the compiled module traces as one

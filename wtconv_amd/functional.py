@@ -197,6 +197,7 @@ class _WTConvFn(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.autograd.function.once_differentiable      # double backward raises instead of being silently wrong
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         x, base_w, base_b, base_s, *wt = ctx.saved_tensors
