@@ -126,6 +126,10 @@ def bench_layer(torch, dev, dtype_name, workload, steps, warmup, per_kernel=True
         "step_frac_valu": 2 * 3 * mac_per_pixel(K, L) * P / (wall_ms * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
         "buffer_sets": nsets,
     }
+    # the roof that binds is the slower of the two (HBM at 8 TB/s, fp32 vector FMA at 78.6
+    # TFLOP/s); the attainment of that roof is the larger of the two fractions
+    res["binding_roof"] = "valu" if res["step_frac_valu"] >= res["step_frac_hbm"] else "hbm"
+    res["step_frac_binding_roof"] = max(res["step_frac_valu"], res["step_frac_hbm"])
     if not per_kernel:
         return res
 
@@ -329,7 +333,7 @@ def main():
                                f"({args.workload}), all parameter grads, seeded default init"},
         "step": {k: main_res[k] for k in ("step_algorithmic_bytes", "step_GBps", "step_frac_hbm", "step_GFLOP",
                                           "step_frac_valu", "ms_per_step_events_median", "ms_per_step_events_min",
-                                          "buffer_sets")},
+                                          "buffer_sets", "binding_roof", "step_frac_binding_roof")},
     }
     if "kernels" in main_res:
         line["kernels"] = main_res["kernels"]
