@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 #endif
 #include <stdint.h>
+#include <type_traits>
 
 #include "../../include/wtconv_hip.h"
 
@@ -153,11 +154,28 @@ __device__ __forceinline__ void pin_values(float (&v)[N]) {
 #endif
 }
 
-// Sum over the 64 lanes of a wavefront; every lane gets the total.
+// Sum over the 64 lanes of a wavefront; every lane gets the total.  On the GPU: six DPP adds
+// (quad permutes, row mirrors, row broadcasts) and one v_readlane, no LDS traffic -- the
+// weight-gradient kernels reduce up to 76 running sums per workgroup this way.
 __device__ __forceinline__ float wave_sum(float v) {
+#ifdef WT_EMULATE
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
   return v;
+#else
+  auto dpp = [](float x, auto ctrl, auto row_mask) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
+                                                      decltype(row_mask)::value, 0xf, false));
+  };
+  using std::integral_constant;
+  v += dpp(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xf>{});    // quad_perm [1,0,3,2]
+  v += dpp(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xf>{});    // quad_perm [2,3,0,1]
+  v += dpp(v, integral_constant<int, 0x141>{}, integral_constant<int, 0xf>{});   // row_half_mirror
+  v += dpp(v, integral_constant<int, 0x140>{}, integral_constant<int, 0xf>{});   // row_mirror: row sums
+  v += dpp(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{});   // row_bcast:15 into rows 1, 3
+  v += dpp(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{});   // row_bcast:31 into rows 2, 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+#endif
 }
 
 }  // namespace wt
