@@ -154,6 +154,18 @@ __device__ __forceinline__ void pin_values(float (&v)[N]) {
 #endif
 }
 
+// Value of lane (lane ^ mask) of the wavefront; `lane4` = 4 * lane, computed once by the
+// caller, so that one exchange costs one integer op and one ds_bpermute (the generic
+// __shfl_xor recomputes and range-checks the source lane every time).
+__device__ __forceinline__ float wave_xor(float v, int lane4, int mask) {
+#ifdef WT_EMULATE
+  (void)lane4;
+  return __shfl_xor(v, mask, kWave);
+#else
+  return __int_as_float(__builtin_amdgcn_ds_bpermute(lane4 ^ (mask << 2), __float_as_int(v)));
+#endif
+}
+
 // Sum over the 64 lanes of a wavefront; every lane gets the total.  On the GPU: six DPP adds
 // (quad permutes, row mirrors, row broadcasts) and one v_readlane, no LDS traffic -- the
 // weight-gradient kernels reduce up to 76 running sums per workgroup this way.

@@ -253,6 +253,7 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
   const int gsh = group_shift(nitem);
   const int s = tid & ((1 << gsh) - 1);
   const int c0 = 4 * s;
+  const int lane4 = (tid & (kWave - 1)) << 2;
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int i = (tid >> gsh) + p * (nthreads >> gsh);
@@ -286,8 +287,8 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
       }
     }
     // level 2: rows i (even) and i+1 of level 1
-    const float bot0 = __shfl_xor(ll1[0], 1 << gsh, kWave);
-    const float bot1 = __shfl_xor(ll1[1], 1 << gsh, kWave);
+    const float bot0 = wave_xor(ll1[0], lane4, 1 << gsh);
+    const float bot1 = wave_xor(ll1[1], lane4, 1 << gsh);
     const bool own2 = valid && (i & 1) == 0;
     float ll2;
     {
@@ -302,9 +303,9 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
       }
     }
     if (fuse >= 3) {   // level 3: level-2 positions (i/2, s), (i/2, s+1), (i/2+1, s), (i/2+1, s+1)
-      const float right = __shfl_xor(ll2, 1, kWave);
-      const float down = __shfl_xor(ll2, 2 << gsh, kWave);
-      const float diag = __shfl_xor(right, 2 << gsh, kWave);
+      const float right = wave_xor(ll2, lane4, 1);
+      const float down = wave_xor(ll2, lane4, 2 << gsh);
+      const float diag = wave_xor(right, lane4, 2 << gsh);
       if (valid && (i & 3) == 0 && (s & 1) == 0) {
         const float sac = ll2 + down, sbd = right + diag, dac = ll2 - down, dbd = right - diag;
         float* o3 = d3 + ((i >> 2) + P1) * str3 + (s >> 1) + P1;
@@ -652,13 +653,13 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
 
   constexpr bool kPrefetch = MODE == 0 || MODE == 3;
   WT_TICK_INIT();
-  zero_lds(lds_all, pl.lds_floats);
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
   {
     int p0, c0;
     locate(blockIdx.x, p0, c0);
     if (kPrefetch && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
   }
+  zero_lds(lds_all, pl.lds_floats);      // while the first plane is on its way from HBM
   WT_LDS_BARRIER();
   WT_TICK(0);
   for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
@@ -868,7 +869,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     for (int t = 0; t < KK; ++t) acc[s][t] = 0.f;
 
   WT_TICK_INIT();
-  zero_lds(lds, pl.lds_floats);
 
   // slot-local bases: level l of slot k starts k*(h_l+P) rows below the top of the stack
   auto a_slot = [&](int l) { return lds + pl.aoff[l] + slot * (pl.h[l] + P) * pl.astr[l]; };
@@ -887,6 +887,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     plane_fetch<T, 1>(x + off, pl.H, pl.W, ltid, nps, xa, xb);
     plane_fetch<T, 1>(g + off, pl.H, pl.W, ltid, nps, ga, gb);
   }
+  zero_lds(lds, pl.lds_floats);          // while the first planes are on their way from HBM
   WT_LDS_BARRIER();
 
   for (int bv = b_begin; bv < b_end; bv += pb) {
