@@ -491,35 +491,31 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
   }
 }
 
-// Store up to N consecutive outputs (4-element vectors when N is a multiple of 4, the
-// destination is aligned to 4 elements and vec4 is set); `nvalid` of them lie inside the row.
+// Store up to N consecutive outputs (`nvalid` of them lie inside the row): 4-element vectors
+// when the whole strip is inside, the destination is aligned to 4 elements and vec4 is set.
 template <typename T, int N>
 __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[N], int nvalid, bool vec4) {
-  if constexpr (N % 4 != 0) {
+  if constexpr (N % 4 == 0) {
+    if (vec4 && nvalid == N) {           // the common case: whole strip inside the row, 16-byte stores
 #pragma unroll
-    for (int e = 0; e < N; ++e)
-      if (e < nvalid) dst[e] = from_f32<T>(v[e]);
-    return;
-  }
-#pragma unroll
-  for (int k = 0; k < N / 4; ++k) {
-    if (vec4 && 4 * k + 4 <= nvalid) {
-      if constexpr (sizeof(T) == 4) {
-        float4 q;
-        q.x = v[4 * k]; q.y = v[4 * k + 1]; q.z = v[4 * k + 2]; q.w = v[4 * k + 3];
-        *reinterpret_cast<float4*>(dst + 4 * k) = q;
-      } else {
-        uint2 q;
-        q.x = static_cast<uint32_t>(f32_to_bf16(v[4 * k])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 1])) << 16);
-        q.y = static_cast<uint32_t>(f32_to_bf16(v[4 * k + 2])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 3])) << 16);
-        *reinterpret_cast<uint2*>(dst + 4 * k) = q;
+      for (int k = 0; k < N / 4; ++k) {
+        if constexpr (sizeof(T) == 4) {
+          float4 q;
+          q.x = v[4 * k]; q.y = v[4 * k + 1]; q.z = v[4 * k + 2]; q.w = v[4 * k + 3];
+          *reinterpret_cast<float4*>(dst + 4 * k) = q;
+        } else {
+          uint2 q;
+          q.x = static_cast<uint32_t>(f32_to_bf16(v[4 * k])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 1])) << 16);
+          q.y = static_cast<uint32_t>(f32_to_bf16(v[4 * k + 2])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 3])) << 16);
+          *reinterpret_cast<uint2*>(dst + 4 * k) = q;
+        }
       }
-    } else {
-#pragma unroll
-      for (int e = 4 * k; e < 4 * k + 4; ++e)
-        if (e < nvalid) dst[e] = from_f32<T>(v[e]);
+      return;
     }
   }
+#pragma unroll
+  for (int e = 0; e < N; ++e)
+    if (e < nvalid) dst[e] = from_f32<T>(v[e]);
 }
 
 // Level 1: conv of the four sub-bands, add Z_2, inverse Haar, add the scaled base conv
@@ -591,6 +587,8 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
     const int r0 = 2 * i, c0 = 2 * j0;
     int nvalid = W - c0;
     if (nvalid > NO) nvalid = NO;
+    pin_values(o0);      // all outputs computed before the stores: keeps the compiler from sinking
+    pin_values(o1);      // the last FMAs behind the store branches and splitting the 16-byte stores
     if (nvalid > 0) {
       store_row<T, NO>(out_plane + r0 * W + c0, o0, nvalid, pl.vec_ok != 0);
       if (r0 + 1 < H) store_row<T, NO>(out_plane + (r0 + 1) * W + c0, o1, nvalid, pl.vec_ok != 0);
@@ -661,6 +659,10 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   }
   zero_lds(lds_all, pl.lds_floats);      // while the first plane is on its way from HBM
   WT_LDS_BARRIER();
+  // Every path into the loop body has now waited for its prefetch (here, and before the stores
+  // of the final phase below), so the commit at the top of the body needs no vmcnt wait of its
+  // own -- which would also wait for the stores of the previous plane.
+  WT_WAIT_VMEM();
   WT_TICK(0);
   for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
     const int u = WT_UNIFORM(uv);
