@@ -2,6 +2,7 @@
 // planning and kernel launches.  Nothing here allocates, frees or synchronises.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "common.h"
@@ -137,6 +138,9 @@ static int run_plane2d_mode(const void* x, void* out, const float* fw, const flo
   const int slots = pl.block / sg;
   const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
   int nwg = compute_units() * resident_per_cu(kern, pl.block, lds);
+#if defined(WT_PHASE_TIMING)
+  if (const char* e = getenv("WT_WG_PER_CU")) nwg = compute_units() * atoi(e);   // profiling aid: occupancy sweep
+#endif
   if (nwg > nunits) nwg = nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(pl.block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");

@@ -75,18 +75,29 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 // wt_phase_ticks[], readable through wtconv_debug_phase_ticks().
 #if defined(WT_PHASE_TIMING) && !defined(WT_EMULATE)
 __device__ unsigned long long wt_phase_ticks[16];
-#define WT_TICK_INIT() long long wt_t_prev = clock64()
+// Thread 0 of every workgroup sums the ticks of each phase in registers and adds them to the
+// global counters once, at WT_TICK_FLUSH() (one atomic per phase and workgroup: no contention
+// that would distort the phases themselves).
+#define WT_TICK_INIT() long long wt_t_prev = clock64(); long long wt_t_acc[16] = {0}
 #define WT_TICK(k)                                                                         \
   do {                                                                                     \
     if (threadIdx.x == 0) {                                                                \
       const long long wt_t_now = clock64();                                                \
-      atomicAdd(&wt_phase_ticks[k], static_cast<unsigned long long>(wt_t_now - wt_t_prev)); \
+      wt_t_acc[k] += wt_t_now - wt_t_prev;                                                 \
       wt_t_prev = wt_t_now;                                                                \
+    }                                                                                      \
+  } while (0)
+#define WT_TICK_FLUSH()                                                                    \
+  do {                                                                                     \
+    if (threadIdx.x == 0) {                                                                \
+      _Pragma("unroll") for (int wt_k = 0; wt_k < 16; ++wt_k)                              \
+        if (wt_t_acc[wt_k]) atomicAdd(&wt_phase_ticks[wt_k], static_cast<unsigned long long>(wt_t_acc[wt_k])); \
     }                                                                                      \
   } while (0)
 #else
 #define WT_TICK_INIT() do {} while (0)
 #define WT_TICK(k) do {} while (0)
+#define WT_TICK_FLUSH() do {} while (0)
 #endif
 
 namespace wt {
@@ -151,6 +162,16 @@ __device__ __forceinline__ void pin_values(float (&v)[N]) {
   for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i]));
 #else
   (void)v;
+#endif
+}
+
+// Product of two indices that fit 24 bits (rows, strides and offsets inside a plane or the
+// LDS): v_mul_i32_i24 runs at full rate, the 32-bit v_mul_lo_u32 at a quarter of it.
+__device__ __forceinline__ int imul(int a, int b) {
+#ifdef WT_EMULATE
+  return a * b;
+#else
+  return __mul24(a, b);
 #endif
 }
 

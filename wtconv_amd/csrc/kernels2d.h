@@ -144,16 +144,16 @@ __device__ __forceinline__ void load_analysis1(const T* __restrict__ src, int H,
     float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
     const bool has_b = 2 * i + 1 < H;
     if (valid) {
-      load4<T>(src + (2 * i) * W + c0, a);
-      if (has_b) load4<T>(src + (2 * i + 1) * W + c0, b);
+      load4<T>(src + imul(2 * i, W) + c0, a);
+      if (has_b) load4<T>(src + imul(2 * i + 1, W) + c0, b);
     }
-    float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+    float* x0 = d0 + imul(2 * i + P0, str0) + c0 + P0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       x0[k] = a[k];
       if (has_b) x0[str0 + k] = b[k];
     }
-    float* o = d1 + (i + P1) * str1 + 2 * s + P1;
+    float* o = d1 + imul(i + P1, str1) + 2 * s + P1;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const float sac = a[2 * t] + b[2 * t], sbd = a[2 * t + 1] + b[2 * t + 1];
@@ -185,8 +185,8 @@ __device__ __forceinline__ void plane_fetch(const T* __restrict__ src, int H, in
       // both loads unconditional (no merge with constants, hence no wait right behind the
       // load); a missing bottom row re-reads the top one and is zeroed in plane_commit
       const int rb = 2 * i + 1 < H ? 2 * i + 1 : 2 * i;
-      load4<T>(src + (2 * i) * W + c0, a[p]);
-      load4<T>(src + rb * W + c0, b[p]);
+      load4<T>(src + imul(2 * i, W) + c0, a[p]);
+      load4<T>(src + imul(rb, W) + c0, b[p]);
     }
   }
 }
@@ -213,13 +213,13 @@ __device__ __forceinline__ void plane_commit(const float (&a)[NP][4], const floa
         aa[k] = valid ? a[p][k] : 0.f;
         bb[k] = (valid && has_b) ? b[p][k] : 0.f;
       }
-      float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+      float* x0 = d0 + imul(2 * i + P0, str0) + c0 + P0;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         x0[k] = aa[k];
         if (has_b) x0[str0 + k] = bb[k];
       }
-      float* o = d1 + (i + P1) * str1 + 2 * s + P1;
+      float* o = d1 + imul(i + P1, str1) + 2 * s + P1;
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const float sac = aa[2 * t] + bb[2 * t], sbd = aa[2 * t + 1] + bb[2 * t + 1];
@@ -266,14 +266,14 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
       bb[k] = (valid && has_b) ? b[p][k] : 0.f;
     }
     if (valid) {
-      float* x0 = d0 + (2 * i + P0) * str0 + c0 + P0;
+      float* x0 = d0 + imul(2 * i + P0, str0) + c0 + P0;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         x0[k] = aa[k];
         if (has_b) x0[str0 + k] = bb[k];
       }
     }
-    float* o1 = d1 + (i + P1) * str1 + 2 * s + P1;
+    float* o1 = d1 + imul(i + P1, str1) + 2 * s + P1;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const float sac = aa[2 * t] + bb[2 * t], sbd = aa[2 * t + 1] + bb[2 * t + 1];
@@ -295,7 +295,7 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
       const float sac = ll1[0] + bot0, sbd = ll1[1] + bot1, dac = ll1[0] - bot0, dbd = ll1[1] - bot1;
       ll2 = own2 ? 0.5f * (sac + sbd) : 0.f;
       if (own2) {
-        float* o2 = d2 + ((i >> 1) + P1) * str2 + s + P1;
+        float* o2 = d2 + imul((i >> 1) + P1, str2) + s + P1;
         o2[0] = ll2;
         o2[pl2] = 0.5f * (dac + dbd);
         o2[2 * pl2] = 0.5f * (sac - sbd);
@@ -308,7 +308,7 @@ __device__ __forceinline__ void plane_commit_fused(const float (&a)[NP][4], cons
       const float diag = wave_xor(right, lane4, 2 << gsh);
       if (valid && (i & 3) == 0 && (s & 1) == 0) {
         const float sac = ll2 + down, sbd = right + diag, dac = ll2 - down, dbd = right - diag;
-        float* o3 = d3 + ((i >> 2) + P1) * str3 + (s >> 1) + P1;
+        float* o3 = d3 + imul((i >> 2) + P1, str3) + (s >> 1) + P1;
         o3[0] = 0.5f * (sac + sbd);
         o3[pl3] = 0.5f * (dac + dbd);
         o3[2 * pl3] = 0.5f * (sac - sbd);
@@ -329,10 +329,10 @@ __device__ __forceinline__ void analysis_level(const float* __restrict__ src, in
   if (rpp == 0) {   // a row is wider than the lane group: plain strided walk
     for (int it = tid; it < hl * wl; it += nthreads) {
       const int i = it / wl, j = it - i * wl;
-      const float* s0 = src + (2 * i + sP) * sstr + 2 * j + sP;
+      const float* s0 = src + imul(2 * i + sP, sstr) + 2 * j + sP;
       const float a = s0[0], b = s0[1], c = s0[sstr], d = s0[sstr + 1];
       const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
-      float* o = dst + (i + dP) * dstr + j + dP;
+      float* o = dst + imul(i + dP, dstr) + j + dP;
       o[0] = 0.5f * (sac + sbd);
       o[dpl] = 0.5f * (dac + dbd);
       o[2 * dpl] = 0.5f * (sac - sbd);
@@ -343,10 +343,10 @@ __device__ __forceinline__ void analysis_level(const float* __restrict__ src, in
   const int j = tid & ((1 << gsh) - 1);
   if (j >= wl) return;
   for (int i = tid >> gsh; i < hl; i += rpp) {
-    const float* s0 = src + (2 * i + sP) * sstr + 2 * j + sP;
+    const float* s0 = src + imul(2 * i + sP, sstr) + 2 * j + sP;
     const float a = s0[0], b = s0[1], c = s0[sstr], d = s0[sstr + 1];
     const float sac = a + c, sbd = b + d, dac = a - c, dbd = b - d;
-    float* o = dst + (i + dP) * dstr + j + dP;
+    float* o = dst + imul(i + dP, dstr) + j + dP;
     o[0] = 0.5f * (sac + sbd);
     o[dpl] = 0.5f * (dac + dbd);
     o[2 * dpl] = 0.5f * (sac - sbd);
@@ -401,44 +401,60 @@ __device__ __forceinline__ void conv_strip(const float* __restrict__ a, int astr
   }
 }
 
-// Adds sub-band s of one coefficient quad into the four reconstructed samples
-// (a b / c d), without the common factor 1/2: rows of the inverse Haar matrix.
-template <int S>
-__device__ __forceinline__ void ihaar_accumulate(float y, float& a, float& b, float& c, float& d) {
-  a += y;
-  if constexpr (S == 0) { b += y; c += y; d += y; }
-  if constexpr (S == 1) { b += y; c -= y; d -= y; }
-  if constexpr (S == 2) { b -= y; c += y; d -= y; }
-  if constexpr (S == 3) { b -= y; c -= y; d += y; }
+// Conv of sub-band S of TJ coefficient quads: one fenced chunk.
+template <int K, int TJ, int VW, int S>
+__device__ __forceinline__ void subband_conv(const float* __restrict__ a, int astr, int apl, wt_uniform_ptr wf,
+                                             float (&y)[TJ]) {
+#pragma unroll
+  for (int t = 0; t < TJ; ++t) y[t] = 0.f;
+  wt_uniform_ptr w = wf + S * K * K;
+  WT_LAUNDER_UNIFORM_PTR(w);
+  conv_strip<K, TJ, VW>(a + S * apl, astr, w, y);
 }
 
-// The four sub-band convolutions of TJ coefficient quads, accumulated straight into the
-// 2 x 2TJ reconstructed samples (scaled by 2), one fenced chunk per sub-band.
-template <int K, int TJ, int VW, int S>
+// The four sub-band convolutions of TJ coefficient quads and the inverse Haar butterflies:
+// o0 / o1 receive the 2 x 2TJ reconstructed samples scaled by 2 (the caller applies the 1/2).
+// Two butterfly stages (LL +- LH as soon as both exist, then +- (HL +- HH)): 8 additions per
+// quad.  One fenced chunk per sub-band bounds the LDS rows in flight.
+template <int K, int TJ, int VW>
 __device__ __forceinline__ void subband_chunks(const float* __restrict__ a, int astr, int apl,
                                                wt_uniform_ptr wf, const float* __restrict__ zin,
                                                float (&o0)[2 * TJ], float (&o1)[2 * TJ]) {
-  if constexpr (S < 4) {
-    float y[TJ];
+  float p[TJ], m[TJ];
+  {
+    float ll[TJ];
+    subband_conv<K, TJ, VW, 0>(a, astr, apl, wf, ll);
+    if (zin != nullptr) {
 #pragma unroll
-    for (int t = 0; t < TJ; ++t) y[t] = 0.f;
-    wt_uniform_ptr w = wf + S * K * K;
-    WT_LAUNDER_UNIFORM_PTR(w);
-    conv_strip<K, TJ, VW>(a + S * apl, astr, w, y);
-    if constexpr (S == 0) {
-      if (zin != nullptr) {
-#pragma unroll
-        for (int t = 0; t < TJ; ++t) y[t] += zin[t];
-      }
+      for (int t = 0; t < TJ; ++t) ll[t] += zin[t];
     }
-#pragma unroll
-    for (int t = 0; t < TJ; ++t)
-      ihaar_accumulate<S>(y[t], o0[2 * t], o0[2 * t + 1], o1[2 * t], o1[2 * t + 1]);
-    pin_values(o0);
-    pin_values(o1);
+    pin_values(ll);
     WT_CHUNK_FENCE();
-    subband_chunks<K, TJ, VW, S + 1>(a, astr, apl, wf, zin, o0, o1);
+    float lh[TJ];
+    subband_conv<K, TJ, VW, 1>(a, astr, apl, wf, lh);
+#pragma unroll
+    for (int t = 0; t < TJ; ++t) { p[t] = ll[t] + lh[t]; m[t] = ll[t] - lh[t]; }
+    pin_values(p);
+    pin_values(m);
+    WT_CHUNK_FENCE();
   }
+  float hl[TJ];
+  subband_conv<K, TJ, VW, 2>(a, astr, apl, wf, hl);
+  pin_values(hl);
+  WT_CHUNK_FENCE();
+  float hh[TJ];
+  subband_conv<K, TJ, VW, 3>(a, astr, apl, wf, hh);
+#pragma unroll
+  for (int t = 0; t < TJ; ++t) {
+    const float q = hl[t] + hh[t], n = hl[t] - hh[t];
+    o0[2 * t] = p[t] + q;
+    o0[2 * t + 1] = p[t] - q;
+    o1[2 * t] = m[t] + n;
+    o1[2 * t + 1] = m[t] - n;
+  }
+  pin_values(o0);
+  pin_values(o1);
+  WT_CHUNK_FENCE();
 }
 
 __device__ __forceinline__ void ihaar4(float ll, float lh, float hl, float hh,
@@ -475,17 +491,15 @@ __device__ __forceinline__ void synth_inner(float* __restrict__ lds, const Plan2
   if ((ltid >> gsh) >= rpp) return;            // more strips than lanes: not used (nth >= 16 >= strips)
   for (int i = ltid >> gsh; i < hl; i += rpp) {
     float o0[2 * TJ], o1[2 * TJ];
-#pragma unroll
-    for (int t = 0; t < 2 * TJ; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
-    subband_chunks<K, TJ, VW, 0>(A + (i - R + P) * astr + (j0 - R + P), astr, apl, wl_f,
-                                 has_carry ? Zin + i * zin_str + j0 : nullptr, o0, o1);
+    subband_chunks<K, TJ, VW>(A + imul(i - R + P, astr) + (j0 - R + P), astr, apl, wl_f,
+                                 has_carry ? Zin + imul(i, zin_str) + j0 : nullptr, o0, o1);
     const int r0 = 2 * i;
 #pragma unroll
     for (int t = 0; t < 2 * TJ; ++t) {
       const int c0 = 2 * j0 + t;
       if (c0 < wo) {
-        Zout[r0 * zout_str + c0] = 0.5f * o0[t];
-        if (r0 + 1 < ho) Zout[(r0 + 1) * zout_str + c0] = 0.5f * o1[t];
+        Zout[imul(r0, zout_str) + c0] = 0.5f * o0[t];
+        if (r0 + 1 < ho) Zout[imul(r0 + 1, zout_str) + c0] = 0.5f * o1[t];
       }
     }
   }
@@ -546,15 +560,13 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
   if ((ltid >> gsh) >= rpp) return;
   for (int i = ltid >> gsh; i < hl; i += rpp) {
     float o0[NO], o1[NO];
-#pragma unroll
-    for (int t = 0; t < NO; ++t) { o0[t] = 0.f; o1[t] = 0.f; }
-    subband_chunks<K, TJ, VW, 0>(A + (i - R + P) * astr + (j0 - R + P), astr, apl, w1_f,
-                                 has_carry ? Zin + i * zin_str + j0 : nullptr, o0, o1);
+    subband_chunks<K, TJ, VW>(A + imul(i - R + P, astr) + (j0 - R + P), astr, apl, w1_f,
+                                 has_carry ? Zin + imul(i, zin_str) + j0 : nullptr, o0, o1);
 #pragma unroll
     for (int t = 0; t < NO; ++t) { o0[t] = fmaf(0.5f, o0[t], bias); o1[t] = fmaf(0.5f, o1[t], bias); }
     // base conv of output rows 2i, 2i+1, columns 2j0 .. 2j0+NO-1, accumulated on top; input
     // row r feeds output row 0 through kernel row r and output row 1 through kernel row r-1
-    const float* xw = X + (2 * i - R + P) * xstr + (2 * j0 - R + P);
+    const float* xw = X + imul(2 * i - R + P, xstr) + (2 * j0 - R + P);
     constexpr int NRX = pad_to(NO + K - 1, VWX);
     wt_uniform_ptr wb = wb_f;
     WT_LAUNDER_UNIFORM_PTR(wb);
@@ -590,8 +602,8 @@ __device__ __forceinline__ void synth_final(float* __restrict__ lds, const Plan2
     pin_values(o0);      // all outputs computed before the stores: keeps the compiler from sinking
     pin_values(o1);      // the last FMAs behind the store branches and splitting the 16-byte stores
     if (nvalid > 0) {
-      store_row<T, NO>(out_plane + r0 * W + c0, o0, nvalid, pl.vec_ok != 0);
-      if (r0 + 1 < H) store_row<T, NO>(out_plane + (r0 + 1) * W + c0, o1, nvalid, pl.vec_ok != 0);
+      store_row<T, NO>(out_plane + imul(r0, W) + c0, o0, nvalid, pl.vec_ok != 0);
+      if (r0 + 1 < H) store_row<T, NO>(out_plane + imul(r0 + 1, W) + c0, o1, nvalid, pl.vec_ok != 0);
     }
   }
 }
@@ -634,29 +646,62 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   const int ppw = sg < kWave ? kWave >> pl.sg_shift : 1;      // planes per wave
   const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
 
-  // plane of this thread in work unit u (-1: none) and its (wave-uniform) channel
-  auto locate = [&](int u, int& plane, int& c) {
+  // Plane of this thread in a work unit (-1: none) and its (wave-uniform) channel.  The
+  // divisions happen once: `locate` positions the state on the workgroup's first unit, and
+  // `advance` moves it by gridDim.x units with additions and one compare (a 32-bit integer
+  // division costs ~35 vector instructions, several of them quarter rate).
+  struct Loc { int plane, c, key, rem; };       // key: un-clamped plane (sg >= 64); rem: gidx % groups (sg < 64)
+  const int G = gridDim.x;
+  int step_c = 0, step_q = 0, step_r = 0;
+  if (sg < kWave) {
+    step_q = (4 * G) / pl.groups_per_channel;
+    step_r = 4 * G - step_q * pl.groups_per_channel;
+  } else {
+    step_c = static_cast<int>((static_cast<long long>(G) * slots) % pl.C);
+  }
+  auto resolve = [&](Loc& s) {
     if (sg < kWave) {
-      const int gidx = u * 4 + wave;
-      c = gidx / pl.groups_per_channel;
-      const int b = (gidx - c * pl.groups_per_channel) * ppw + ((tid & (kWave - 1)) >> pl.sg_shift);
-      plane = (c < pl.C && b < pl.B) ? b * pl.C + c : -1;
-      if (c >= pl.C) c = pl.C - 1;
+      const int b = imul(s.rem, ppw) + ((tid & (kWave - 1)) >> pl.sg_shift);
+      s.plane = (s.c < pl.C && b < pl.B) ? imul(b, pl.C) + s.c : -1;
     } else {
-      plane = u * slots + slot;
-      if (plane >= pl.nplanes) plane = -1;
-      c = plane >= 0 ? plane % pl.C : 0;
+      s.plane = s.key < pl.nplanes ? s.key : -1;
     }
   };
+  auto locate = [&](int u, Loc& s) {
+    if (sg < kWave) {
+      const int gidx = u * 4 + wave;
+      s.c = gidx / pl.groups_per_channel;
+      s.rem = gidx - s.c * pl.groups_per_channel;
+      s.key = 0;
+    } else {
+      s.key = u * slots + slot;
+      s.c = s.key % pl.C;
+      s.rem = 0;
+    }
+    resolve(s);
+  };
+  auto advance = [&](Loc& s) {
+    if (sg < kWave) {
+      s.c += step_q;
+      s.rem += step_r;
+      if (s.rem >= pl.groups_per_channel) { s.rem -= pl.groups_per_channel; s.c += 1; }
+    } else {
+      s.key += G * slots;           // may pass nplanes: resolve() maps that to "no plane"
+      s.c += step_c;
+      if (s.c >= pl.C) s.c -= pl.C;
+    }
+    resolve(s);
+  };
+  // the channel used for the weights (clamped: a thread without a plane still runs uniform code)
+  auto channel_of = [&](const Loc& s) { return s.c < pl.C ? s.c : pl.C - 1; };
 
   constexpr bool kPrefetch = MODE == 0 || MODE == 3;
   WT_TICK_INIT();
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
-  {
-    int p0, c0;
-    locate(blockIdx.x, p0, c0);
-    if (kPrefetch && p0 >= 0) plane_fetch<T, kFetchPasses>(x + p0 * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
-  }
+  Loc nxt;
+  locate(blockIdx.x, nxt);
+  if (kPrefetch && nxt.plane >= 0)
+    plane_fetch<T, kFetchPasses>(x + nxt.plane * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
   zero_lds(lds_all, pl.lds_floats);      // while the first plane is on its way from HBM
   WT_LDS_BARRIER();
   // Every path into the loop body has now waited for its prefetch (here, and before the stores
@@ -666,10 +711,10 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   WT_TICK(0);
   for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
     const int u = WT_UNIFORM(uv);
-    int plane, cv;
-    locate(u, plane, cv);
-    const int c = WT_UNIFORM(cv);
+    const int plane = nxt.plane;
+    const int c = WT_UNIFORM(channel_of(nxt));
     const bool live = plane >= 0;
+    advance(nxt);
     wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * KK);
     const size_t plane_off = static_cast<size_t>(live ? plane : 0) * plane_elems;
     int l0 = 2;
@@ -696,11 +741,8 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     }
     WT_LDS_BARRIER();
     WT_TICK(1);
-    if (kPrefetch && u + static_cast<int>(gridDim.x) < nunits) {
-      int pn, cn;
-      locate(u + gridDim.x, pn, cn);
-      if (pn >= 0) plane_fetch<T, kFetchPasses>(x + pn * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
-    }
+    if (kPrefetch && u + static_cast<int>(gridDim.x) < nunits && nxt.plane >= 0)
+      plane_fetch<T, kFetchPasses>(x + nxt.plane * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
     for (int lv = l0; lv <= pl.L; ++lv) {
       const int l = WT_UNIFORM(lv);
       if (live)
@@ -721,6 +763,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     WT_LDS_BARRIER();   // the next plane overwrites the buffers read above
     WT_TICK(7);
   }
+  WT_TICK_FLUSH();
 }
 
 // ------------------------------------------------------------------ parameter gradients
@@ -817,17 +860,17 @@ __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr
     const int npair = (h + 1) >> 1;
     for (int ip = pass_row0 * rpp + (lane >> gsh); ip < npair; ip += pass_step * rpp) {
       const int i = 2 * ip;
-      const float* gy = G + i * gstr + j0;
+      const float* gy = G + imul(i, gstr) + j0;
 #pragma unroll
       for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t] + gy[gstr + t], gsum);
-      corr_strip2<K, TJ, VW>(A + i * astr + j0, astr, gy, gy + gstr, acc);
+      corr_strip2<K, TJ, VW>(A + imul(i, astr) + j0, astr, gy, gy + gstr, acc);
     }
   } else {
     for (int i = pass_row0 * rpp + (lane >> gsh); i < h; i += pass_step * rpp) {
-      const float* gy = G + i * gstr + j0;
+      const float* gy = G + imul(i, gstr) + j0;
 #pragma unroll
       for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t], gsum);
-      corr_strip<K, TJ, VW>(A + i * astr + j0, astr, gy, acc);   // A already points R rows/cols up-left
+      corr_strip<K, TJ, VW>(A + imul(i, astr) + j0, astr, gy, acc);   // A already points R rows/cols up-left
     }
   }
 }
@@ -996,6 +1039,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
   }
   WT_LDS_BARRIER();
   WT_TICK(13);
+  WT_TICK_FLUSH();
   float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * (NF * KK + 1);
   for (int o = tid; o < NF * KK + 1; o += blockDim.x) {
     float v = 0.f;
