@@ -194,6 +194,59 @@ def test_under_autocast_and_channels_last(hip_device):
     U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
 
 
+def _random_cases(kind, n, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        K = rng.choice([1, 3, 5, 5, 7])
+        L = rng.randint(1, 5)
+        B, C = rng.randint(1, 5), rng.randint(1, 6)
+        if kind == "2d":
+            big = rng.random() < 0.15
+            H = rng.randint(120, 180) if big else rng.randint(1, 70)
+            W = rng.randint(120, 180) if big else rng.randint(1, 70)
+            if big:
+                B, C = min(B, 2), min(C, 2)
+            shape = (B, C, H, W)
+        else:
+            N = rng.choice([rng.randint(1, 300), rng.randint(300, 5000), rng.randint(5000, 20000)])
+            shape = (B, C, N)
+        cases.append((shape, K, L, rng.random() < 0.8))
+    return cases
+
+
+@pytest.mark.parametrize("kind,seed", [("2d", 11), ("1d", 12)])
+def test_random_shapes_against_oracle(hip_device, kind, seed):
+    """Seeded random sweep over kernel sizes, levels and (mostly odd) sizes: every dispatch
+    path (packed small planes, plane-resident, level-by-level; tiled and row-resident 1-D)
+    is hit by some case; all of out, grad_x and parameter gradients are compared."""
+    for shape, K, L, bias in _random_cases(kind, 24, seed):
+        try:
+            _run_fp32(kind, shape[1], K, L, shape, hip_device, bias=bias, seed=seed)
+        except AssertionError as e:
+            raise AssertionError(f"{kind} shape={shape} K={K} L={L} bias={bias}: {e}") from e
+
+
+@pytest.mark.parametrize("kind,seed", [("2d", 31), ("1d", 32)])
+def test_random_shapes_bf16_against_oracle(hip_device, kind, seed):
+    """The same sweep with bf16 activations (fp32 parameters), against fp32 maths on the
+    bf16-rounded inputs."""
+    W2, W1 = _mods()
+    rb = lambda t: t.to(torch.bfloat16).float()
+    for shape, K, L, bias in _random_cases(kind, 16, seed):
+        ref, x, g = U.seeded_case(kind, shape[1], K, L, shape, bias=bias, seed=seed)
+        U.randomize_scales(ref)
+        x, g = rb(x), rb(g)
+        mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, K, L, bias=bias)
+        got = U.hip_run(mod, x, g, hip_device, dtype=torch.bfloat16)
+        want = U.oracle_run(ref, x, g, torch.float32)
+        try:
+            U.compare_all(got, want, U.assert_bf16)
+        except AssertionError as e:
+            raise AssertionError(f"{kind} bf16 shape={shape} K={K} L={L} bias={bias}: {e}") from e
+
+
 def test_double_backward_raises(hip_device):
     W2, _ = _mods()
     mod = W2(4, 4, 3, wt_levels=1).to(hip_device)
