@@ -30,8 +30,10 @@ def build(force=False):
     return EXE
 
 
-def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600):
-    """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays."""
+def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600, lds_limit=None):
+    """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays.
+    `lds_limit` (bytes) lowers the LDS budget of the dispatch, so that small planes take the
+    level-by-level kernels that real runs only use for planes beyond 160 KB."""
     exe = build()
     if dims == 2:
         B, C, H, W = x.shape
@@ -57,6 +59,9 @@ def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, 
         env = dict(os.environ)
         env["ASAN_OPTIONS"] = "detect_leaks=0"
         env.pop("LD_PRELOAD", None)
+        env.pop("WT_EMU_LDS_LIMIT", None)
+        if lds_limit is not None:
+            env["WT_EMU_LDS_LIMIT"] = str(int(lds_limit))
         r = subprocess.run([exe, fin, fout], capture_output=True, text=True, timeout=timeout, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"emu_driver failed ({r.returncode}):\n{r.stderr[-4000:]}")

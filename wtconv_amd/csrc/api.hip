@@ -214,14 +214,21 @@ static int run_wgrad2d_k(int K, int L, const void* x, const void* g, float* part
 }
 
 // ---- planes that do not fit LDS: level-by-level kernels through an HBM pyramid ----------
+static size_t lds_fit_limit() {
+#ifdef WT_EMULATE   // host emulation only: send small planes through the level-by-level kernels
+  if (const char* e = getenv("WT_EMU_LDS_LIMIT")) return static_cast<size_t>(atol(e));
+#endif
+  return kLdsLimitBytes;
+}
+
 static bool plane_fits_lds(int B, int C, int H, int W, int K, int L) {
   Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, 4, nullptr, nullptr, nullptr);
-  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= kLdsLimitBytes;
+  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= lds_fit_limit();
 }
 
 static bool wgrad_fits_lds(int B, int C, int H, int W, int K, int L) {
   Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, 4, nullptr, nullptr, nullptr, 1);
-  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= kLdsLimitBytes;
+  return static_cast<size_t>(pl.plane_lds_floats) * 4 <= lds_fit_limit();
 }
 
 static size_t round_up64(size_t v) { return (v + 63) / 64 * 64; }
@@ -246,16 +253,21 @@ static Stream2D make_stream2d(int B, int C, int H, int W, int L) {
   return s;
 }
 
-// Batch chunks of the streamed weight-gradient kernels: about 2048 workgroups per launch of
-// the four sub-band filters of a level (a constant rule: workspace sizes do not depend on the device).
-static void stream_chunks(int B, int C, int* bchunk, int* nchunk) {
-  int want = (2048 + 4 * C - 1) / (4 * C);
+// Chunks of the streamed weight-gradient kernels: the (batch item, tile) units of a level are
+// split over `nchunk` workgroups per filter, about 2048 workgroups for the base-conv launch
+// (C filters) and four times that for the sub-band launches, never more chunks than the
+// finest level has units (a constant rule: workspace sizes do not depend on the device).
+static int stream_chunks(int B, int C, int H, int W) {
+  const long units = static_cast<long>(B) * ((H + kStreamTile - 1) / kStreamTile) *
+                     ((W + kStreamTileW - 1) / kStreamTileW);
+  long want = (2048 + C - 1) / C;
+  if (want > 64) want = 64;
+  if (want > units) want = units;
   if (want < 1) want = 1;
-  if (want > B) want = B;
-  const int bc = (B + want - 1) / want;
-  *bchunk = bc;
-  *nchunk = (B + bc - 1) / bc;
+  return static_cast<int>(want);
 }
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <typename T>
 static int stream_analysis_chain(const T* src, float* pyr, const Stream2D& sp, hipStream_t stream) {
@@ -283,20 +295,23 @@ static int run_stream2d(const void* x_, void* out_, const float* fw, const float
   T* out = static_cast<T*>(out_);
   if (int e = stream_analysis_chain<T>(x, pyr, sp, stream)) return e;
   const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
+  const unsigned gz = (sp.nplanes + gy - 1) / gy;
   const int NF = 1 + 4 * sp.L;
   for (int l = sp.L; l >= 1; --l) {
     const unsigned tiles = static_cast<unsigned>(((sp.h[l] + kStreamTile - 1) / kStreamTile) *
-                                                 ((sp.w[l] + kStreamTile - 1) / kStreamTile));
+                                                 ((sp.w[l] + kStreamTileW - 1) / kStreamTileW));
     const float* zin = l < sp.L ? pyr + sp.zoff[l + 1] : nullptr;
+    const bool io_ok = l > 1 || (aligned16(x) && aligned16(out));
+    const int vec = (sp.w[l] % 4 == 0 && aligned16(pyr) ? 1 : 0) | (sp.w[l - 1] % 4 == 0 && io_ok ? 2 : 0);
     if (l > 1) {
-      WT_LAUNCH((stream_synth_kernel<T, K, false>), dim3(tiles, gy), dim3(256), 0, stream,
+      WT_LAUNCH((stream_synth_kernel<T, K, false>), dim3(tiles, gy, gz), dim3(256), 0, stream,
                 static_cast<const float*>(pyr + sp.aoff[l]), sp.h[l], sp.w[l], zin, pyr + sp.zoff[l], sp.h[l - 1],
                 sp.w[l - 1], static_cast<const T*>(nullptr), static_cast<T*>(nullptr), fw, fb, sp.C, NF,
-                1 + 4 * (l - 1), sp.nplanes);
+                1 + 4 * (l - 1), sp.nplanes, vec);
     } else {
-      WT_LAUNCH((stream_synth_kernel<T, K, true>), dim3(tiles, gy), dim3(256), 0, stream,
+      WT_LAUNCH((stream_synth_kernel<T, K, true>), dim3(tiles, gy, gz), dim3(256), 0, stream,
                 static_cast<const float*>(pyr + sp.aoff[1]), sp.h[1], sp.w[1], zin, static_cast<float*>(nullptr), sp.H,
-                sp.W, x, out, fw, fb, sp.C, NF, 1, sp.nplanes);
+                sp.W, x, out, fw, fb, sp.C, NF, 1, sp.nplanes, vec);
     }
     if (int e = check_launch("stream_synth_kernel")) return e;
   }
@@ -317,21 +332,30 @@ static int run_stream2d_k(int K, const void* x, void* out, const float* fw, cons
 
 template <typename T, int K>
 static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, float* pyr_x, float* pyr_g,
-                              const Stream2D& sp, int B, int bchunk, int nchunk, hipStream_t stream) {
+                              const Stream2D& sp, int B, int nchunk, hipStream_t stream) {
   const T* x = static_cast<const T*>(x_);
   const T* g = static_cast<const T*>(g_);
   if (int e = stream_analysis_chain<T>(x, pyr_x, sp, stream)) return e;
   if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream)) return e;
   const int rec = (1 + 4 * sp.L) * K * K + 1;
-  WT_LAUNCH((stream_corr_kernel<T, K>), dim3(sp.C, nchunk), dim3(256), 0, stream, x, g,
+  const bool pyr_ok = aligned16(pyr_x) && aligned16(pyr_g);
+  // chunks of a launch: at least four (batch item, tile) units per workgroup where the level has them
+  auto level_chunks = [&](int h, int w) {
+    const long units = static_cast<long>(B) * ((h + kStreamTile - 1) / kStreamTile) *
+                       ((w + kStreamTileW - 1) / kStreamTileW);
+    const long nc = units / 4;
+    return static_cast<unsigned>(nc < 1 ? 1 : (nc > nchunk ? nchunk : nc));
+  };
+  WT_LAUNCH((stream_corr_kernel<T, K>), dim3(sp.C, level_chunks(sp.H, sp.W)), dim3(256), 0, stream, x, g,
             static_cast<size_t>(sp.H) * sp.W, static_cast<size_t>(0), sp.H, sp.W, partial, rec, 0, 1, 1, B, sp.C,
-            bchunk);
+            (sp.W % 4 == 0 && aligned16(x) && aligned16(g)) ? 1 : 0, nchunk);
   if (int e = check_launch("stream_corr_kernel")) return e;
   for (int l = 1; l <= sp.L; ++l) {
     const size_t n = static_cast<size_t>(sp.h[l]) * sp.w[l];
-    WT_LAUNCH((stream_corr_kernel<float, K>), dim3(sp.C * 4, nchunk), dim3(256), 0, stream,
+    WT_LAUNCH((stream_corr_kernel<float, K>), dim3(sp.C * 4, level_chunks(sp.h[l], sp.w[l])), dim3(256), 0, stream,
               static_cast<const float*>(pyr_x + sp.aoff[l]), static_cast<const float*>(pyr_g + sp.aoff[l]), 4 * n, n,
-              sp.h[l], sp.w[l], partial, rec, 1 + 4 * (l - 1), 4, 0, B, sp.C, bchunk);
+              sp.h[l], sp.w[l], partial, rec, 1 + 4 * (l - 1), 4, 0, B, sp.C,
+              (sp.w[l] % 4 == 0 && pyr_ok) ? 1 : 0, nchunk);
     if (int e = check_launch("stream_corr_kernel")) return e;
   }
   return 0;
@@ -339,12 +363,12 @@ static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, fl
 
 template <typename T>
 static int run_stream2d_wgrad_k(int K, const void* x, const void* g, float* partial, float* pyr_x, float* pyr_g,
-                                const Stream2D& sp, int B, int bchunk, int nchunk, hipStream_t stream) {
+                                const Stream2D& sp, int B, int nchunk, hipStream_t stream) {
   switch (K) {
-    case 1: return run_stream2d_wgrad<T, 1>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
-    case 3: return run_stream2d_wgrad<T, 3>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
-    case 5: return run_stream2d_wgrad<T, 5>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
-    case 7: return run_stream2d_wgrad<T, 7>(x, g, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+    case 1: return run_stream2d_wgrad<T, 1>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
+    case 3: return run_stream2d_wgrad<T, 3>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
+    case 5: return run_stream2d_wgrad<T, 5>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
+    case 7: return run_stream2d_wgrad<T, 7>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
   }
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
@@ -622,7 +646,7 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
       wgrad_chunks(B, C, wgrad_planes_per_iter(B, H, W, K, levels), kWgradResident, &bchunk, &nchunk);
       floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
     } else {      // partial sums, then the pyramids of x and of grad_out
-      stream_chunks(B, C, &bchunk, &nchunk);
+      nchunk = stream_chunks(B, C, H, W);
       floats = round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1)) +
                2 * make_stream2d(B, C, H, W, levels).floats;
     }
@@ -683,13 +707,13 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
                             : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
   } else {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
-    stream_chunks(B, C, &bchunk, &nchunk);
+    nchunk = stream_chunks(B, C, H, W);
     if (nchunk > 65535 || C > 0x7fffffff / 4) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
     float* pyr_x = partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * L) * K * K + 1));
     float* pyr_g = pyr_x + sp.floats;
     e = dtype == WTCONV_F32
-            ? run_stream2d_wgrad_k<float>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream)
-            : run_stream2d_wgrad_k<bf16_t>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, bchunk, nchunk, stream);
+            ? run_stream2d_wgrad_k<float>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream)
+            : run_stream2d_wgrad_k<bf16_t>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
   }
   if (e) return e;
   GradTable gt = {};

@@ -1074,6 +1074,7 @@ __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchun
   const int c = blockIdx.x;
   for (int o = threadIdx.x; o < NF * KK; o += blockDim.x) {
     float sum = 0.f;
+#pragma unroll 8                       // several chunk loads in flight; the order of the adds is unchanged
     for (int ch = 0; ch < nchunk; ++ch) sum += partial[(static_cast<size_t>(ch) * C + c) * stride + o];
     const int f = o / KK, t = o - f * KK;
     float gam, wv;
@@ -1097,6 +1098,7 @@ __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchun
     if (o == 0) {
       // sumG sits in the last slot of the channel's partial record
       float sg = 0.f;
+#pragma unroll 8
       for (int ch = 0; ch < nchunk; ++ch) sg += partial[(static_cast<size_t>(ch) * C + c) * stride + NF * KK];
       if (p.base_bias != nullptr) {
         dot = fmaf(load_param(p.base_bias, pdtype, c), sg, dot);
