@@ -281,6 +281,67 @@ def test_torch_compile_custom_op(hip_device):
                 assert torch.equal(p.grad, eager[n]), n
 
 
+def test_hip_graph_replay_matches_eager(hip_device):
+    """A whole training step (forward, input gradient, parameter gradients) captured in a HIP
+    graph: the library allocates nothing, clears nothing with memset nodes and never
+    synchronises, so the capture holds only its kernels.  Every replay, with new input values
+    and eager work of the same layer between the replays, must equal the eager result
+    bit for bit, and the first replay must also match the oracle."""
+    W2, W1 = _mods()
+    for kind, cls, shape, L in (("2d", W2, (3, 6, 28, 28), 3), ("1d", W1, (3, 6, 1024), 4)):
+        ref, x, g = U.seeded_case(kind, 6, 5, L, shape)
+        U.randomize_scales(ref)
+        mod = U.copy_to_hip_module(ref, cls, kind, 5, L).to(hip_device)
+        params = [(n, p) for n, p in mod.named_parameters() if p.requires_grad]
+        xs = x.to(hip_device).requires_grad_(True)
+        gs = g.to(hip_device)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):                      # warm-up outside the capture
+                xs.grad = None
+                for _, p in params:
+                    p.grad = None
+                mod(xs).backward(gs)
+            xs.grad = None
+            for _, p in params:
+                p.grad = None
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                out = mod(xs)
+                out.backward(gs)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        gen = torch.Generator().manual_seed(7)
+        for it in range(4):
+            xn = x if it == 0 else torch.randn(*shape, generator=gen)
+            gn = g if it == 0 else torch.randn(*g.shape, generator=gen)
+            with torch.no_grad():
+                xs.copy_(xn.to(hip_device))
+                gs.copy_(gn.to(hip_device))
+            graph.replay()
+            torch.cuda.synchronize()
+            got_out, got_dx = out.detach().clone(), xs.grad.clone()
+            got = {n: p.grad.clone() for n, p in params}
+            held = {n: p.grad for n, p in params}   # the graph's own gradient buffers
+            for _, p in params:
+                p.grad = None
+            xe = xn.to(hip_device).requires_grad_(True)
+            oe = mod(xe)                            # eager work between the replays
+            oe.backward(gn.to(hip_device))
+            torch.cuda.synchronize()
+            assert torch.equal(got_out, oe.detach()) and torch.equal(got_dx, xe.grad), (kind, it)
+            for n, p in params:
+                assert torch.equal(got[n], p.grad), (kind, it, n)
+                p.grad = held[n]
+            if it == 0:
+                wo, wdx, wg = U.oracle_run(ref, x, g, torch.float64)
+                U.assert_fp32(got_out.cpu(), wo, "out")
+                U.assert_fp32(got_dx.cpu(), wdx, "grad_x")
+                for n in got:
+                    U.assert_fp32(got[n].cpu(), wg[n], n)
+
+
 # ------------------------------------------------------------------ full-size checks
 def test_config2_full_size_fp32(hip_device):
     """WTConv2d(96,96,5,wt_levels=3) on x[128,96,56,56]: forward/input-gradient planes are
