@@ -21,6 +21,7 @@
 #define WT_SCHED_FENCE() do {} while (0)
 #define WT_UNIFORM(x) (x)
 #define WT_LDS_BARRIER() __syncthreads()
+#define WT_WAVE_LDS_SYNC() __syncthreads()
 #define WT_WAIT_VMEM() do {} while (0)
 #define WT_CHUNK_FENCE() do {} while (0)
 #define WT_LAUNDER_UNIFORM_PTR(p) do {} while (0)
@@ -45,6 +46,15 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");     \
     __builtin_amdgcn_s_barrier();                                       \
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");     \
+  } while (0)
+// Orders the LDS traffic of one wave only: lanes of a wave that exchange data through LDS (a
+// plane owned by 64 lanes or fewer) need no workgroup barrier, because the LDS instructions of a
+// wave execute in issue order; this only keeps the compiler from moving them across.
+#define WT_WAVE_LDS_SYNC()                                              \
+  do {                                                                  \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");     \
+    __builtin_amdgcn_wave_barrier();                                    \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");     \
   } while (0)
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt left at their maxima).
 // gfx950 counts loads and stores in the same counter; waiting for the prefetch loads

@@ -81,6 +81,13 @@ __global__ void fold_params_kernel(ParamTable p, int pdtype, float* __restrict__
   }
 }
 
+// Synchronisation between the phases of a plane: workgroup barrier, or only the ordering of
+// one wave's LDS traffic when every plane belongs to the lanes of a single wave.
+__device__ __forceinline__ void plane_sync(bool wave_local) {
+  if (wave_local) WT_WAVE_LDS_SYNC();
+  else WT_LDS_BARRIER();
+}
+
 // ------------------------------------------------------------------ plane load
 // Copy one contiguous H x W plane from HBM into a haloed (or padded) LDS buffer whose
 // element (r, col) sits at dst[(r + P) * str + col + P].
@@ -708,6 +715,9 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   // of the final phase below), so the commit at the top of the body needs no vmcnt wait of its
   // own -- which would also wait for the stores of the previous plane.
   WT_WAIT_VMEM();
+  // A plane owned by the lanes of one wave needs no workgroup barrier between its phases: the
+  // waves of the workgroup drift apart and fill each other's latency-bound phases.
+  const bool wave_local = pl.sg_shift <= 6;
   WT_TICK(0);
   for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
     const int u = WT_UNIFORM(uv);
@@ -739,7 +749,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
       if (live) load_plane<T>(x + plane_off, lds + pl.aoff[0], pl.H, pl.W, pl.astr[0], pl.P, ltid, sg);
       l0 = 1;
     }
-    WT_LDS_BARRIER();
+    plane_sync(wave_local);
     WT_TICK(1);
     if (kPrefetch && u + static_cast<int>(gridDim.x) < nunits && nxt.plane >= 0)
       plane_fetch<T, kFetchPasses>(x + nxt.plane * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
@@ -748,19 +758,19 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
       if (live)
         analysis_level(lds + pl.aoff[l - 1], pl.astr[l - 1], pl.P, lds + pl.aoff[l], pl.astr[l], pl.apl[l], pl.P,
                        pl.h[l], pl.w[l], ltid, sg);
-      WT_LDS_BARRIER();
+      plane_sync(wave_local);
     }
     WT_TICK(2);
     for (int lv = pl.L; lv >= 2; --lv) {
       const int l = WT_UNIFORM(lv);
       if (live) synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK, ltid, sg);
-      WT_LDS_BARRIER();
+      plane_sync(wave_local);
       WT_TICK(1 + l);
     }
     WT_WAIT_VMEM();     // next plane's loads have landed; the stores below are not waited for
     WT_WAVE_PRIORITY(0);
     if (live) synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off, ltid, sg);
-    WT_LDS_BARRIER();   // the next plane overwrites the buffers read above
+    plane_sync(wave_local);   // the next plane overwrites the buffers read above
     WT_TICK(7);
   }
   WT_TICK_FLUSH();
