@@ -886,6 +886,7 @@ __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr
 }
 
 constexpr int wgrad_sets(int L) { return L >= 4 ? 3 : (L >= 2 ? 2 : 1); }
+constexpr int kStripMinWidth = 12;   // coarse levels of the weight-gradient kernel: strips from this width on
 
 template <typename T, int K, int L, int TJ>
 __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
@@ -1016,8 +1017,15 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       const int l = role_a ? 3 : 2;
       if (l <= L) {
         float unused = 0.f;
-        corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0, 1,
-                                   acc[1], 0.f, unused);
+        // a level at least kStripMinWidth wide is walked in row pairs of TJ-wide strips like the
+        // first set (one pass of a wave instead of four at 14 x 14), a narrower one by single
+        // coefficients (more lanes busy)
+        if (pl.w[l] >= kStripMinWidth)
+          corr_level<K, TJ, VW, true>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0,
+                                      1, acc[1], 0.f, unused);
+        else
+          corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0,
+                                     1, acc[1], 0.f, unused);
       }
     }
     if constexpr (NSET >= 3) {                 // set 2: level 5 (A) / level 4 (B)
