@@ -123,13 +123,30 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
 
-// round-to-nearest-even, NaN kept quiet
+// round-to-nearest-even, NaN kept quiet.  On the device this is the hardware conversion
+// (v_cvt_pk_bf16_f32, one instruction per two values); the host emulation spells it out.
+#ifdef WT_EMULATE
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   uint32_t u = __float_as_uint(f);
   if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
   u += 0x7fffu + ((u >> 16) & 1u);
   return static_cast<bf16_t>(u >> 16);
 }
+// two values in one 32-bit word, `lo` in the low half
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+}
+#else
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  return __builtin_bit_cast(bf16_t, static_cast<__bf16>(f));
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float wt_f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 wt_bf16x2 __attribute__((ext_vector_type(2)));
+  const wt_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, wt_bf16x2));
+}
+#endif
 
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }

@@ -113,10 +113,10 @@ __device__ __forceinline__ void store_run(T* __restrict__ dst, const float (&v)[
 #pragma unroll
       for (int k = 0; k < N / 8; ++k) {
         uint4 q;
-        q.x = static_cast<uint32_t>(f32_to_bf16(v[8 * k])) | (static_cast<uint32_t>(f32_to_bf16(v[8 * k + 1])) << 16);
-        q.y = static_cast<uint32_t>(f32_to_bf16(v[8 * k + 2])) | (static_cast<uint32_t>(f32_to_bf16(v[8 * k + 3])) << 16);
-        q.z = static_cast<uint32_t>(f32_to_bf16(v[8 * k + 4])) | (static_cast<uint32_t>(f32_to_bf16(v[8 * k + 5])) << 16);
-        q.w = static_cast<uint32_t>(f32_to_bf16(v[8 * k + 6])) | (static_cast<uint32_t>(f32_to_bf16(v[8 * k + 7])) << 16);
+        q.x = pack_bf16x2(v[8 * k], v[8 * k + 1]);
+        q.y = pack_bf16x2(v[8 * k + 2], v[8 * k + 3]);
+        q.z = pack_bf16x2(v[8 * k + 4], v[8 * k + 5]);
+        q.w = pack_bf16x2(v[8 * k + 6], v[8 * k + 7]);
         reinterpret_cast<uint4*>(dst)[k] = q;
       }
     }

@@ -205,8 +205,7 @@ __device__ __forceinline__ void row1d_unstage(T* __restrict__ row, const float* 
         uint32_t qq[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          qq[k] = static_cast<uint32_t>(f32_to_bf16(vals[2 * k])) |
-                  (static_cast<uint32_t>(f32_to_bf16(vals[2 * k + 1])) << 16);
+          qq[k] = pack_bf16x2(vals[2 * k], vals[2 * k + 1]);
         q.x = qq[0]; q.y = qq[1]; q.z = qq[2]; q.w = qq[3];
       }
       *reinterpret_cast<uint4*>(row + p) = q;

@@ -526,8 +526,8 @@ __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[
           *reinterpret_cast<float4*>(dst + 4 * k) = q;
         } else {
           uint2 q;
-          q.x = static_cast<uint32_t>(f32_to_bf16(v[4 * k])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 1])) << 16);
-          q.y = static_cast<uint32_t>(f32_to_bf16(v[4 * k + 2])) | (static_cast<uint32_t>(f32_to_bf16(v[4 * k + 3])) << 16);
+          q.x = pack_bf16x2(v[4 * k], v[4 * k + 1]);
+          q.y = pack_bf16x2(v[4 * k + 2], v[4 * k + 3]);
           *reinterpret_cast<uint2*>(dst + 4 * k) = q;
         }
       }
