@@ -859,7 +859,7 @@ __device__ __forceinline__ void corr_strip2(const float* __restrict__ a, int ast
 template <int K, int TJ, int VW, bool PAIR>
 __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr, const float* __restrict__ G,
                                            int gstr, int h, int w, int lane, int pass_row0, int pass_step,
-                                           float (&acc)[K * K], float gmul, float& gsum) {
+                                           float (&acc)[K * K]) {
   const int nstrip = (w + TJ - 1) / TJ;
   const int gsh = group_shift(nstrip);
   const int strip = lane & ((1 << gsh) - 1);
@@ -871,15 +871,11 @@ __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr
     for (int ip = pass_row0 * rpp + (lane >> gsh); ip < npair; ip += pass_step * rpp) {
       const int i = 2 * ip;
       const float* gy = G + imul(i, gstr) + j0;
-#pragma unroll
-      for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t] + gy[gstr + t], gsum);
       corr_strip2<K, TJ, VW>(A + imul(i, astr) + j0, astr, gy, gy + gstr, acc);
     }
   } else {
     for (int i = pass_row0 * rpp + (lane >> gsh); i < h; i += pass_step * rpp) {
       const float* gy = G + imul(i, gstr) + j0;
-#pragma unroll
-      for (int t = 0; t < TJ; ++t) gsum = fmaf(gmul, gy[t], gsum);
       corr_strip<K, TJ, VW>(A + imul(i, astr) + j0, astr, gy, acc);   // A already points R rows/cols up-left
     }
   }
@@ -1009,31 +1005,35 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     {
       const int l = role_a ? 0 : 1;            // set 0, strips of TJ: base conv rows (A) / level 1 (B)
       corr_level<K, TJ, VW, true>(a_plane(l, role_a ? 0 : q), pl.astr[l], g_plane(l, role_a ? 0 : q), pl.gstr[l],
-                            rows(l), pl.w[l], lane, role_a ? q : 0, role_a ? 4 : 1, acc[0], role_a ? 1.f : 0.f,
-                            gsum);
+                            rows(l), pl.w[l], lane, role_a ? q : 0, role_a ? 4 : 1, acc[0]);
+    }
+    if (wave == 0) {
+      // bias gradient: the sum of grad_out is 2^L times the sum of its coarsest LL band (every
+      // Haar level halves the sum of a plane; padding, gap rows and absent planes hold zeros)
+      const float* GL = g_plane(L, 0);
+      const int n = imul(rows(L), pl.gstr[L]);
+      for (int e = lane; e < n; e += kWave) gsum += GL[e];
     }
     WT_TICK(10);
     if constexpr (NSET >= 2) {                 // set 1, single coefficients: level 3 (A) / level 2 (B)
       const int l = role_a ? 3 : 2;
       if (l <= L) {
-        float unused = 0.f;
         // a level at least kStripMinWidth wide is walked in row pairs of TJ-wide strips like the
         // first set (one pass of a wave instead of four at 14 x 14), a narrower one by single
         // coefficients (more lanes busy)
         if (pl.w[l] >= kStripMinWidth)
           corr_level<K, TJ, VW, true>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0,
-                                      1, acc[1], 0.f, unused);
+                                      1, acc[1]);
         else
           corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0,
-                                     1, acc[1], 0.f, unused);
+                                     1, acc[1]);
       }
     }
     if constexpr (NSET >= 3) {                 // set 2: level 5 (A) / level 4 (B)
       const int l = role_a ? 5 : 4;
       if (l <= L) {
-        float unused = 0.f;
         corr_level<K, 1, 1, false>(a_plane(l, q), pl.astr[l], g_plane(l, q), pl.gstr[l], rows(l), pl.w[l], lane, 0, 1,
-                                   acc[2], 0.f, unused);
+                                   acc[2]);
       }
     }
     WT_TICK(11);
@@ -1052,7 +1052,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       if (lane == 0) red[wave * NRED + s * KK + t] = v;
     }
   {
-    const float v = wave_sum(gsum);
+    const float v = wave_sum(gsum) * static_cast<float>(1 << L);
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
   WT_LDS_BARRIER();
