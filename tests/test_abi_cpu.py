@@ -40,6 +40,7 @@ def test_workspace_sizes(lib):
     assert par >= 4 * C * ((1 + 4 * L) * K * K + 1)
     assert lib.wtconv1d_workspace_bytes(64, 64, 4096, 5, 4, 0) >= 4 * (64 * 9 * 5 + 64)
     assert lib.wtconv2d_workspace_bytes(0, C, 56, 56, K, L, 0) == 0
+    assert lib.wtconv2d_workspace_bytes(1, 1, 20000, 20000, K, L, 0) == 0     # plane beyond 2^28 elements
     # planes whose pyramid exceeds LDS: the workspace also holds the fp32 pyramid(s)
     big = lib.wtconv2d_workspace_bytes(2, 4, 400, 400, K, L, 0)
     assert big >= 4 * 2 * 4 * (400 * 400 + 200 * 200 * 4 // 4)
@@ -67,6 +68,7 @@ def _params(L=2):
     (dict(x=0), -1, "null"),
     (dict(H=400, W=400), -3, "workspace"),     # larger than LDS: the HBM pyramid needs a larger workspace
     (dict(ws_bytes=16), -3, "workspace"),
+    (dict(H=20000, W=20000), -2, "2^28"),      # 32-bit offsets inside a plane
 ])
 def test_forward_argument_validation(lib, kw, code, needle):
     """Bad arguments are rejected with a code and a message before any kernel launch."""

@@ -234,6 +234,7 @@ static bool wgrad_fits_lds(int B, int C, int H, int W, int K, int L) {
 }
 
 static size_t round_up64(size_t v) { return (v + 63) / 64 * 64; }
+constexpr long long kMaxPlaneElems = 1LL << 28;
 
 static Stream2D make_stream2d(int B, int C, int H, int W, int L) {
   Stream2D s = {};
@@ -380,6 +381,8 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
                         void* stream_, int flip) {
   if (int e = check_common(fn, params, B, C, K, L, dtype, pdtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
+  if (static_cast<long long>(H) * W > kMaxPlaneElems)   // 32-bit offsets inside a plane and its four stacked sub-bands
+    return fail(WTCONV_E_UNSUPPORTED, "%s: a plane of %dx%d exceeds 2^28 elements", fn, H, W);
   if (x == nullptr || out == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
@@ -641,6 +644,7 @@ int wtconv_debug_phase_ticks(unsigned long long* out16, int reset) {
 
 size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
   if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
+  if (static_cast<long long>(H) * W > kMaxPlaneElems) return 0;
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     int bchunk, nchunk;
@@ -681,6 +685,8 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   const int L = levels;
   if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
+  if (static_cast<long long>(H) * W > kMaxPlaneElems)   // 32-bit offsets inside a plane and its four stacked sub-bands
+    return fail(WTCONV_E_UNSUPPORTED, "%s: a plane of %dx%d exceeds 2^28 elements", fn, H, W);
   if (x == nullptr || grad_out == nullptr || grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
   if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
       (params->base_bias != nullptr && grads->base_bias == nullptr))
