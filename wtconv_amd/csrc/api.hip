@@ -131,9 +131,7 @@ static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float
 template <typename T, int K, int TJ1, int MODE>
 static int run_plane2d_mode(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
                             hipStream_t stream) {
-  // planes narrow enough for single-coefficient strips at level 1 have one or two coefficients per
-  // row at the coarser levels: single strips there too keep more lanes busy
-  auto kern = wt2d_plane_kernel<T, K, TJ1, (TJ1 == 1 ? 1 : kTJC), MODE>;
+  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC, MODE>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   const int sg = 1 << pl.sg_shift;

@@ -12,7 +12,8 @@ namespace wt {
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Strip widths of the 2-D kernels (outputs per work item along a row).
-constexpr int kTJC = 2;     // coarser levels of the plane kernel
+constexpr int kTJC = 1;     // coarser levels of the plane kernel: single coefficients keep the most lanes busy
+                            // (measured against strips of 2: 28x28 planes 106 -> 100 us, 14x14 73 -> 71, 56x56 equal)
 constexpr int kTJW = 4;     // weight-gradient correlation strips
 
 inline int pow2_ceil(int v) { int p = 1; while (p < v) p *= 2; return p; }
