@@ -26,8 +26,8 @@ VALU_PEAK_TFLOPS = 78.6         # fp32 vector FMA without packed-FP32 code gener
 # run), scaled by what a plain device copy of one activation tensor reads on the same
 # counters (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); see profiles/wt2d_stage1_fp32_hbm_traffic.txt.
 MEASURED_TRAFFIC_BYTES = {
-    ("stage1", "fp32", "wt2d_plane_kernel"): (151070 + 150528) * 1024,
-    ("stage1", "fp32", "wt2d_wgrad_kernel"): (301768 + 1583) * 1024,
+    ("stage1", "fp32", "wt2d_plane_kernel"): (151061 + 150528) * 1024,
+    ("stage1", "fp32", "wt2d_wgrad_kernel"): (301756 + 1583) * 1024,
 }
 
 WORKLOADS = {
