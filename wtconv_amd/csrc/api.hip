@@ -270,17 +270,22 @@ static int stream_chunks(int B, int C, int H, int W) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// `ll_only`: the level-1 detail bands are not stored (forward / input-gradient pass: its last
+// synthesis level rebuilds them from the pixels; the weight-gradient pass needs them).
 template <typename T>
-static int stream_analysis_chain(const T* src, float* pyr, const Stream2D& sp, hipStream_t stream) {
+static int stream_analysis_chain(const T* src, float* pyr, const Stream2D& sp, hipStream_t stream, bool ll_only) {
   const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
   for (int l = 1; l <= sp.L; ++l) {
     const int n = sp.h[l] * sp.w[l];
     const unsigned gx = static_cast<unsigned>((n + 255) / 256);
-    if (l == 1) {
-      WT_LAUNCH(stream_analysis_kernel<T>, dim3(gx, gy), dim3(256), 0, stream, src,
+    if (l == 1 && ll_only) {
+      WT_LAUNCH((stream_analysis_kernel<T, true>), dim3(gx, gy), dim3(256), 0, stream, src,
+                static_cast<size_t>(sp.H) * sp.W, sp.H, sp.W, pyr + sp.aoff[1], sp.h[1], sp.w[1], sp.nplanes);
+    } else if (l == 1) {
+      WT_LAUNCH((stream_analysis_kernel<T, false>), dim3(gx, gy), dim3(256), 0, stream, src,
                 static_cast<size_t>(sp.H) * sp.W, sp.H, sp.W, pyr + sp.aoff[1], sp.h[1], sp.w[1], sp.nplanes);
     } else {
-      WT_LAUNCH(stream_analysis_kernel<float>, dim3(gx, gy), dim3(256), 0, stream,
+      WT_LAUNCH((stream_analysis_kernel<float, false>), dim3(gx, gy), dim3(256), 0, stream,
                 static_cast<const float*>(pyr + sp.aoff[l - 1]), static_cast<size_t>(4) * sp.h[l - 1] * sp.w[l - 1],
                 sp.h[l - 1], sp.w[l - 1], pyr + sp.aoff[l], sp.h[l], sp.w[l], sp.nplanes);
     }
@@ -294,7 +299,9 @@ static int run_stream2d(const void* x_, void* out_, const float* fw, const float
                         hipStream_t stream) {
   const T* x = static_cast<const T*>(x_);
   T* out = static_cast<T*>(out_);
-  if (int e = stream_analysis_chain<T>(x, pyr, sp, stream)) return e;
+  if (sp.L > 1) {      // a single level is synthesised from the pixels alone
+    if (int e = stream_analysis_chain<T>(x, pyr, sp, stream, true)) return e;
+  }
   const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
   const unsigned gz = (sp.nplanes + gy - 1) / gy;
   const int NF = 1 + 4 * sp.L;
@@ -336,8 +343,8 @@ static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, fl
                               const Stream2D& sp, int B, int nchunk, hipStream_t stream) {
   const T* x = static_cast<const T*>(x_);
   const T* g = static_cast<const T*>(g_);
-  if (int e = stream_analysis_chain<T>(x, pyr_x, sp, stream)) return e;
-  if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream)) return e;
+  if (int e = stream_analysis_chain<T>(x, pyr_x, sp, stream, false)) return e;
+  if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream, false)) return e;
   const int rec = (1 + 4 * sp.L) * K * K + 1;
   const bool pyr_ok = aligned16(pyr_x) && aligned16(pyr_g);
   // chunks of a launch: at least four (batch item, tile) units per workgroup where the level has them

@@ -29,7 +29,7 @@ struct Stream2D {
 // One analysis level: src = x / grad_out (element type TS) or the LL band of the level above
 // (fp32, plane stride 4*hs*ws); reading one past an odd source size returns the zero padding
 // the reference applies (wtconv2d.py:49-51).  grid = (tiles, planes <= 65535), block = 256.
-template <typename TS>
+template <typename TS, bool LL_ONLY>
 __global__ void stream_analysis_kernel(const TS* __restrict__ src, size_t src_plane_stride, int hs, int ws,
                                        float* __restrict__ dst, int hd, int wd, int nplanes) {
   const int n = hd * wd;
@@ -46,9 +46,11 @@ __global__ void stream_analysis_kernel(const TS* __restrict__ src, size_t src_pl
       const float e = (r1 && c1) ? to_f32<TS>(p[ws + 1]) : 0.f;
       const float sac = a + c, sbd = b + e, dac = a - c, dbd = b - e;
       d[q] = 0.5f * (sac + sbd);
-      d[n + q] = 0.5f * (dac + dbd);
-      d[2 * n + q] = 0.5f * (sac - sbd);
-      d[3 * n + q] = 0.5f * (dac - dbd);
+      if constexpr (!LL_ONLY) {            // the forward pass rebuilds the level-1 detail bands from x itself
+        d[n + q] = 0.5f * (dac + dbd);
+        d[2 * n + q] = 0.5f * (sac - sbd);
+        d[3 * n + q] = 0.5f * (dac - dbd);
+      }
     }
   }
 }
@@ -127,30 +129,63 @@ __device__ __forceinline__ void lds_read12(const float* __restrict__ p, float (&
   }
 }
 
-// Tiles of the synthesis kernel: the four sub-bands of the level (haloed, VA elements per
-// load) and, for the last level, the input pixels under them (VO elements per load).  All
-// loads are issued before the first LDS write.
+// Tiles of the synthesis kernel.  Levels >= 2: the four sub-bands of the level (haloed, VA
+// elements per load) from the pyramid.  Last level: only the input pixels under the haloed
+// coefficient tile (VO elements per load); the level-1 sub-bands are rebuilt from them in LDS
+// (haar_tile), which saves reading -- and, in the analysis kernel, writing -- three quarters of
+// the level-1 pyramid.
 template <typename T, int K, bool FINAL, int VA, int VO>
 __device__ __forceinline__ void synth_stage_tiles(const float* __restrict__ Ap, size_t n, int hl, int wl,
                                                   const T* __restrict__ xp, int ho, int wo, int i0, int j0,
                                                   float* __restrict__ At, float* __restrict__ Xt, int tid) {
   constexpr int R = K / 2;
   constexpr int TH = kStreamTile, TW = kStreamTileW, HP = kStreamPad;
-  WindowStage<float, 4, TH + 2 * R, TW + 2 * HP, VA> sa;
-  sa.fetch(Ap, n, hl, wl, i0 - R, j0 - HP, tid);
   if constexpr (FINAL) {
-    WindowStage<T, 1, 2 * TH + 2 * R, 2 * TW + 2 * HP, VO> sx;
-    sx.fetch(xp, 0, ho, wo, 2 * i0 - R, 2 * j0 - HP, tid);
-    sa.commit(At, tid);
+    WindowStage<T, 1, 2 * (TH + 2 * R), 2 * (TW + 2 * HP), VO> sx;
+    sx.fetch(xp, 0, ho, wo, 2 * (i0 - R), 2 * (j0 - HP), tid);
     sx.commit(Xt, tid);
   } else {
+    WindowStage<float, 4, TH + 2 * R, TW + 2 * HP, VA> sa;
+    sa.fetch(Ap, n, hl, wl, i0 - R, j0 - HP, tid);
     sa.commit(At, tid);
   }
 }
 
+// Level-1 Haar analysis of a pixel tile in LDS: coefficient (rr, cc) of the AH x AWD tile comes
+// from pixels (2rr .. 2rr+1, 2cc .. 2cc+1) of the 2AH x 2AWD pixel tile.  Pixels outside the
+// plane were staged as zeros, which is both the zero padding of odd sizes and the zero halo of
+// the sub-band convs (a coefficient outside the level has all four pixels outside the plane).
+template <int AH, int AWD>
+__device__ __forceinline__ void haar_tile(const float* __restrict__ Xt, float* __restrict__ At, int tid) {
+  constexpr int XWD = 2 * AWD;
+  constexpr int PAIRS = AWD / 2;             // two coefficients (four pixels of each row) per step
+  for (int e = tid; e < AH * PAIRS; e += 256) {
+    const int rr = e / PAIRS, cp = e - rr * PAIRS;
+    const float4 top = *reinterpret_cast<const float4*>(Xt + (2 * rr) * XWD + 4 * cp);
+    const float4 bot = *reinterpret_cast<const float4*>(Xt + (2 * rr + 1) * XWD + 4 * cp);
+    const float a[2] = {top.x, top.z}, b[2] = {top.y, top.w}, c[2] = {bot.x, bot.z}, d[2] = {bot.y, bot.w};
+    float o[4][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {            // same operation order as stream_analysis_kernel
+      const float sac = a[t] + c[t], sbd = b[t] + d[t], dac = a[t] - c[t], dbd = b[t] - d[t];
+      o[0][t] = 0.5f * (sac + sbd);
+      o[1][t] = 0.5f * (dac + dbd);
+      o[2][t] = 0.5f * (sac - sbd);
+      o[3][t] = 0.5f * (dac - dbd);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      float* dst = At + (s * AH + rr) * AWD + 2 * cp;
+      dst[0] = o[s][0];
+      dst[1] = o[s][1];
+    }
+  }
+}
+
 // Synthesis of level l: the four sub-band convs of a tile of 16 x 64 coefficients, + Z_{l+1},
-// inverse Haar, cropped.  FINAL (l = 1) adds the scaled base conv and bias of the 32 x 128
-// pixels and stores the layer output; otherwise the result goes to Z_l.  A thread owns four
+// inverse Haar, cropped.  FINAL (l = 1) takes its sub-bands from the input pixels (`A` unused),
+// adds the scaled base conv and bias of the 32 x 128 pixels and stores the layer output;
+// otherwise the sub-bands come from the pyramid and the result goes to Z_l.  A thread owns four
 // adjacent coefficients of a row (2 x 8 output pixels): every LDS row it reads as 16-byte
 // vectors feeds 4K (sub-bands) or 8K (base conv) products.  The tiles carry a column halo of
 // 4 so that their rows start at multiples of 4 elements of the source row.
@@ -168,7 +203,7 @@ __global__ __launch_bounds__(256, 3) void stream_synth_kernel(const float* __res
   constexpr int R = K / 2;
   constexpr int TH = kStreamTile, TW = kStreamTileW, HP = kStreamPad, TJ = 4;
   constexpr int AH = TH + 2 * R, AWD = TW + 2 * HP;
-  constexpr int XH = 2 * TH + 2 * R, XWD = 2 * TW + 2 * HP;
+  constexpr int XH = 2 * AH, XWD = 2 * AWD;   // last level: the pixels under the haloed coefficient tile
   __shared__ alignas(16) float At[4 * AH * AWD];
   __shared__ alignas(16) float Xt[FINAL ? XH * XWD : 4];
   const int tiles_x = (wl + TW - 1) / TW;
@@ -192,6 +227,10 @@ __global__ __launch_bounds__(256, 3) void stream_synth_kernel(const float* __res
       else synth_stage_tiles<T, K, FINAL, 1, 1>(Ap, n, hl, wl, xp, ho, wo, i0, j0, At, Xt, tid);
     }
     __syncthreads();
+    if constexpr (FINAL) {
+      haar_tile<AH, AWD>(Xt, At, tid);
+      __syncthreads();
+    }
     const int i = i0 + r, j = j0 + c0;
     if (i < hl && j < wl) {
       wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(ch) * NF * K * K);
@@ -242,7 +281,7 @@ __global__ __launch_bounds__(256, 3) void stream_synth_kernel(const float* __res
 #pragma unroll
         for (int xr = 0; xr < K + 1; ++xr) {
           float v[16];
-          const float* rowp = Xt + (2 * r + xr) * XWD + 2 * c0;
+          const float* rowp = Xt + (2 * r + xr + R) * XWD + 2 * c0 + HP;
           {
             float lo[12];
             lds_read12(rowp, lo);
