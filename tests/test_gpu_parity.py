@@ -67,6 +67,8 @@ def test_stage_shapes_fp32_small_batch(hip_device, C, H, L):
     ((1, 2, 131, 137), 7, 4, False),   # the same with odd sizes at every level, K = 7
     ((2, 2, 200, 200), 3, 5, True),    # five levels on a large plane
     ((2, 4, 100, 100), 5, 2, True),    # plane-resident forward, level-by-level weight gradients
+    ((1, 2, 160, 192), 5, 1, True),    # a single level on a large plane: synthesised from the pixels alone
+    ((1, 2, 144, 136), 1, 2, False),   # K = 1 on a large plane
 ])
 def test_edge_shapes_fp32(hip_device, shape, K, L, bias):
     _run_fp32("2d", shape[1], K, L, shape, hip_device, bias=bias, seed=3)
