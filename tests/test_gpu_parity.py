@@ -69,6 +69,8 @@ def test_stage_shapes_fp32_small_batch(hip_device, C, H, L):
     ((2, 4, 100, 100), 5, 2, True),    # plane-resident forward, level-by-level weight gradients
     ((1, 2, 160, 192), 5, 1, True),    # a single level on a large plane: synthesised from the pixels alone
     ((1, 2, 144, 136), 1, 2, False),   # K = 1 on a large plane
+    ((1, 1, 3, 3), 7, 4, True),        # one tiny plane, K = 7: the final weight-gradient reduction needs more LDS than the pyramids
+    ((1, 1, 1, 1), 7, 1, True),
 ])
 def test_edge_shapes_fp32(hip_device, shape, K, L, bias):
     _run_fp32("2d", shape[1], K, L, shape, hip_device, bias=bias, seed=3)
@@ -194,6 +196,44 @@ def test_under_autocast_and_channels_last(hip_device):
         half_in = mod(xd.bfloat16())          # bf16 activations, fp32 parameters
     assert half_in.dtype == torch.bfloat16
     U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
+
+
+@pytest.mark.parametrize("kind,shape,L", [("2d", (2, 8, 20, 22), 2), ("1d", (2, 4, 300), 3)])
+def test_fp16_activations(hip_device, kind, shape, L):
+    """float16 activations (the default AMP dtype of the reference's trainer, train.py:180,438):
+    oracle = fp32 maths on the fp16-rounded inputs; bar = rounding of the result to fp16
+    (rtol 2e-3, atol 2e-3 of the oracle's RMS); parameter gradients, which stay fp32, to the fp32 bar."""
+    W2, W1 = _mods()
+    ref, x, g = U.seeded_case(kind, shape[1], 5, L, shape)
+    U.randomize_scales(ref)
+    rh = lambda t: t.to(torch.float16).float()
+    x, g = rh(x), rh(g)
+    mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, 5, L)
+    out, dx, grads = U.hip_run(mod, x, g, hip_device, dtype=torch.float16)
+    wo, wdx, wg = U.oracle_run(ref, x, g, torch.float64)
+
+    def close16(a, b, name):
+        rms = b.double().pow(2).mean().sqrt().item()
+        torch.testing.assert_close(a.double(), b.double(), rtol=2e-3, atol=2e-3 * rms, msg=lambda m: f"{name}: {m}")
+    close16(out, wo, "out")
+    close16(dx, wdx, "grad_x")
+    for n, v in grads.items():
+        U.assert_fp32(v, wg[n], n)
+
+
+def test_fp16_under_autocast(hip_device):
+    """torch.autocast(float16) with an fp16 input, as a WTConvNeXt block sees it under --amp."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 8, 5, 2, (2, 8, 14, 14))
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 2).to(hip_device)
+    xh = x.to(hip_device).half().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = mod(xh)
+    assert out.dtype == torch.float16
+    out.backward(g.to(hip_device).half())
+    assert xh.grad.dtype == torch.float16
+    want = mod(xh.detach().float())
+    torch.testing.assert_close(out.float(), want, rtol=2e-3, atol=2e-3)
 
 
 def _random_cases(kind, n, seed):

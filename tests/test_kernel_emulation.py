@@ -97,6 +97,17 @@ def test_emulated_2d_level_by_level(B, C, H, W, K, L, bias, limit):
     _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
 
 
+# A single tiny plane: the pyramids take less LDS than the final reduction of the
+# weight-gradient kernel ([8 waves][sets * K * K + 1] floats), which the plan must cover.
+@pytest.mark.parametrize("B,C,H,W,K,L", [
+    (1, 1, 1, 1, 7, 4), (1, 1, 2, 2, 7, 5), (1, 1, 4, 4, 7, 2), (1, 1, 1, 1, 7, 1), (1, 1, 1, 1, 5, 2),
+])
+def test_emulated_2d_tiny_plane_reduction_fits_lds(B, C, H, W, K, L):
+    x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, True)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, K)
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
+
+
 def test_emulated_2d_bf16_io_and_params():
     x, g, bw, bb, bs, ws, ss = _case2d(1, 2, 8, 12, 5, 2, True, dtype=1, pdtype=1)
     got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, 5, dtype=1, pdtype=1)

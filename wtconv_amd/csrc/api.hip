@@ -5,6 +5,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <functional>
+#include <mutex>
+#include <unordered_map>
+
 #include "common.h"
 #include "kernels1d.h"
 #include "kernels1d_row.h"
@@ -37,13 +41,41 @@ static int check_launch(const char* what) {
   if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
   return 0;
 }
-// Workgroups above 64 KiB of dynamic LDS need the opt-in attribute.
+// Per-kernel facts that cost a driver call (hundreds of nanoseconds to microseconds each) are
+// looked up once per (device, kernel, launch shape) and kept for the life of the process.
+struct KernelKey {
+  int dev; const void* fn; int block; size_t lds;
+  bool operator==(const KernelKey& o) const { return dev == o.dev && fn == o.fn && block == o.block && lds == o.lds; }
+};
+struct KernelKeyHash {
+  size_t operator()(const KernelKey& k) const {
+    return std::hash<const void*>()(k.fn) ^ (static_cast<size_t>(k.dev) * 0x9e3779b97f4a7c15ull) ^
+           (k.lds * 31 + static_cast<size_t>(k.block));
+  }
+};
+static std::mutex g_kernel_cache_mutex;
+static std::unordered_map<KernelKey, int, KernelKeyHash> g_lds_allowed, g_resident;
+
+static int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); dev = 0; }
+  return dev;
+}
+
+// Workgroups above 64 KiB of dynamic LDS need the opt-in attribute (set once per kernel and size).
 template <typename F> static int allow_lds(F kernel, size_t bytes) {
   if (bytes <= 64 * 1024) return 0;
+  const KernelKey key = {current_device(), reinterpret_cast<const void*>(kernel), 0, bytes};
+  {
+    std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
+    if (g_lds_allowed.count(key)) return 0;
+  }
   const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
                                            static_cast<int>(bytes));
   if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
+  g_lds_allowed[key] = 1;
   return 0;
 }
 #endif
@@ -74,12 +106,20 @@ static int resident_per_cu(F kernel, int block, size_t lds_bytes) {
   (void)kernel; (void)block; (void)lds_bytes;
   return 1;
 #else
+  const KernelKey key = {current_device(), reinterpret_cast<const void*>(kernel), block, lds_bytes};
+  {
+    std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
+    auto it = g_resident.find(key);
+    if (it != g_resident.end()) return it->second;
+  }
   int n = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kernel), block, lds_bytes) !=
           hipSuccess || n < 1) {
     (void)hipGetLastError();
     n = resident_workgroups(1, lds_bytes, block / 64, 8);
   }
+  std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
+  g_resident[key] = n;
   return n;
 #endif
 }
@@ -138,9 +178,6 @@ static int run_plane2d_mode(const void* x, void* out, const float* fw, const flo
   const int slots = pl.block / sg;
   const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
   int nwg = compute_units() * resident_per_cu(kern, pl.block, lds);
-#if defined(WT_PHASE_TIMING)
-  if (const char* e = getenv("WT_WG_PER_CU")) nwg = compute_units() * atoi(e);   // profiling aid: occupancy sweep
-#endif
   if (nwg > nunits) nwg = nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(pl.block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
@@ -632,21 +669,6 @@ const char* wtconv_last_error(void) { return g_err; }
 
 int wtconv_max_kernel_size(void) { return 7; }
 
-#if defined(WT_PHASE_TIMING) && !defined(WT_EMULATE)
-// Profiling aid, only in -DWT_PHASE_TIMING builds: copies (and optionally clears) the 16
-// per-phase tick counters.  Synchronises the device.
-int wtconv_debug_phase_ticks(unsigned long long* out16, int reset) {
-  if (hipDeviceSynchronize() != hipSuccess) return WTCONV_E_LAUNCH;
-  if (out16 && hipMemcpyFromSymbol(out16, HIP_SYMBOL(wt_phase_ticks), 16 * sizeof(unsigned long long)) != hipSuccess)
-    return WTCONV_E_LAUNCH;
-  if (reset) {
-    unsigned long long z[16] = {0};
-    if (hipMemcpyToSymbol(HIP_SYMBOL(wt_phase_ticks), z, sizeof(z)) != hipSuccess) return WTCONV_E_LAUNCH;
-  }
-  return 0;
-}
-#endif
-
 size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
   if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
   if (static_cast<long long>(H) * W > kMaxPlaneElems) return 0;
@@ -714,7 +736,7 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   if (wgrad_fits_lds(B, C, H, W, K, L)) {
     const int pb = wgrad_planes_per_iter(B, H, W, K, L);
     Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
-    finish_wgrad_plan(&pl);
+    finish_wgrad_plan(&pl, K);
     wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
     e = dtype == WTCONV_F32 ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
                             : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);

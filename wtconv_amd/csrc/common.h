@@ -80,36 +80,6 @@ typedef const float __attribute__((address_space(4)))* wt_uniform_ptr;
 #define WT_WAVE_PRIORITY(n) __builtin_amdgcn_s_setprio(n)
 #endif
 
-// Optional profiling aid (off in the product build): -DWT_PHASE_TIMING makes wave 0 of
-// every workgroup add the shader-clock ticks it spent in each kernel phase to
-// wt_phase_ticks[], readable through wtconv_debug_phase_ticks().
-#if defined(WT_PHASE_TIMING) && !defined(WT_EMULATE)
-__device__ unsigned long long wt_phase_ticks[16];
-// Thread 0 of every workgroup sums the ticks of each phase in registers and adds them to the
-// global counters once, at WT_TICK_FLUSH() (one atomic per phase and workgroup: no contention
-// that would distort the phases themselves).
-#define WT_TICK_INIT() long long wt_t_prev = clock64(); long long wt_t_acc[16] = {0}
-#define WT_TICK(k)                                                                         \
-  do {                                                                                     \
-    if (threadIdx.x == 0) {                                                                \
-      const long long wt_t_now = clock64();                                                \
-      wt_t_acc[k] += wt_t_now - wt_t_prev;                                                 \
-      wt_t_prev = wt_t_now;                                                                \
-    }                                                                                      \
-  } while (0)
-#define WT_TICK_FLUSH()                                                                    \
-  do {                                                                                     \
-    if (threadIdx.x == 0) {                                                                \
-      _Pragma("unroll") for (int wt_k = 0; wt_k < 16; ++wt_k)                              \
-        if (wt_t_acc[wt_k]) atomicAdd(&wt_phase_ticks[wt_k], static_cast<unsigned long long>(wt_t_acc[wt_k])); \
-    }                                                                                      \
-  } while (0)
-#else
-#define WT_TICK_INIT() do {} while (0)
-#define WT_TICK(k) do {} while (0)
-#define WT_TICK_FLUSH() do {} while (0)
-#endif
-
 namespace wt {
 
 constexpr int kMaxLevels = WTCONV_MAX_LEVELS;

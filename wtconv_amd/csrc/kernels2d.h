@@ -703,7 +703,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   auto channel_of = [&](const Loc& s) { return s.c < pl.C ? s.c : pl.C - 1; };
 
   constexpr bool kPrefetch = MODE == 0 || MODE == 3;
-  WT_TICK_INIT();
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
   Loc nxt;
   locate(blockIdx.x, nxt);
@@ -718,7 +717,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   // A plane owned by the lanes of one wave needs no workgroup barrier between its phases: the
   // waves of the workgroup drift apart and fill each other's latency-bound phases.
   const bool wave_local = pl.sg_shift <= 6;
-  WT_TICK(0);
   for (int uv = blockIdx.x; uv < nunits; uv += gridDim.x) {
     const int u = WT_UNIFORM(uv);
     const int plane = nxt.plane;
@@ -750,7 +748,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
       l0 = 1;
     }
     plane_sync(wave_local);
-    WT_TICK(1);
     if (kPrefetch && u + static_cast<int>(gridDim.x) < nunits && nxt.plane >= 0)
       plane_fetch<T, kFetchPasses>(x + nxt.plane * plane_elems, pl.H, pl.W, ltid, sg, fa, fbuf);
     for (int lv = l0; lv <= pl.L; ++lv) {
@@ -760,20 +757,16 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
                        pl.h[l], pl.w[l], ltid, sg);
       plane_sync(wave_local);
     }
-    WT_TICK(2);
     for (int lv = pl.L; lv >= 2; --lv) {
       const int l = WT_UNIFORM(lv);
       if (live) synth_inner<K, TJC>(lds, pl, l, fwc + (1 + 4 * (l - 1)) * KK, ltid, sg);
       plane_sync(wave_local);
-      WT_TICK(1 + l);
     }
     WT_WAIT_VMEM();     // next plane's loads have landed; the stores below are not waited for
     WT_WAVE_PRIORITY(0);
     if (live) synth_final<T, K, TJ1>(lds, pl, fwc, fwc + KK, fb[c], out + plane_off, ltid, sg);
     plane_sync(wave_local);   // the next plane overwrites the buffers read above
-    WT_TICK(7);
   }
-  WT_TICK_FLUSH();
 }
 
 // ------------------------------------------------------------------ parameter gradients
@@ -920,7 +913,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
 #pragma unroll
     for (int t = 0; t < KK; ++t) acc[s][t] = 0.f;
 
-  WT_TICK_INIT();
 
   // slot-local bases: level l of slot k starts k*(h_l+P) rows below the top of the stack
   auto a_slot = [&](int l) { return lds + pl.aoff[l] + slot * (pl.h[l] + P) * pl.astr[l]; };
@@ -981,7 +973,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       l0 = 1;
     }
     WT_LDS_BARRIER();
-    WT_TICK(8);
     if (pl.prefetch && has_slot && b0 + pb < b_end) {
       const bool nvalid = b0 + pb + slot < b_end;
       const size_t off = (static_cast<size_t>(nvalid ? b0 + pb + slot : b0) * pl.C + c) * plane_elems;
@@ -998,7 +989,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       }
       WT_LDS_BARRIER();
     }
-    WT_TICK(9);
     WT_WAVE_PRIORITY(0);
     // Both roles run the same code on different planes (one code path keeps a single
     // register set for the sums).
@@ -1014,7 +1004,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
       const int n = imul(rows(L), pl.gstr[L]);
       for (int e = lane; e < n; e += kWave) gsum += GL[e];
     }
-    WT_TICK(10);
     if constexpr (NSET >= 2) {                 // set 1, single coefficients: level 3 (A) / level 2 (B)
       const int l = role_a ? 3 : 2;
       if (l <= L) {
@@ -1036,9 +1025,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
                                    acc[2]);
       }
     }
-    WT_TICK(11);
     WT_LDS_BARRIER();
-    WT_TICK(12);
   }
 
   // cross-lane reduction, then cross-wave through LDS (pyramid buffers are dead now)
@@ -1056,8 +1043,6 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
   WT_LDS_BARRIER();
-  WT_TICK(13);
-  WT_TICK_FLUSH();
   float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * (NF * KK + 1);
   for (int o = tid; o < NF * KK + 1; o += blockDim.x) {
     float v = 0.f;

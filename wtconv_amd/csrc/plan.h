@@ -128,7 +128,11 @@ inline int wgrad_planes_per_iter(int B, int H, int W, int K, int L) {
 }
 
 // Completes a plan for the weight-gradient kernel: threads per stacked plane, prefetch.
-inline void finish_wgrad_plan(Plan2D* pl) {
+inline void finish_wgrad_plan(Plan2D* pl, int K) {
+  // the final reduction reuses the LDS as [8 waves][sets * K * K + 1] floats, which is more
+  // than the pyramids of a single tiny plane take
+  const int red_floats = round_up(8 * (wgrad_sets(pl->L) * K * K + 1), 4);
+  if (pl->lds_floats < red_floats) pl->lds_floats = red_floats;
   const int slots = pow2_ceil(pl->pb);
   pl->slot_shift = log2_int(512 / slots);
   const int nps = 512 / slots;

@@ -63,8 +63,8 @@ def _check_input(x, ndim, what):
         raise ValueError(f"{what} expects a {ndim}-D input, got shape {tuple(x.shape)}")
     if not x.is_cuda:
         raise RuntimeError(f"{what} runs on the GPU only (got a {x.device} tensor); there is no CPU path")
-    if x.dtype not in _DT:
-        raise TypeError(f"{what} supports float32 and bfloat16 activations, got {x.dtype}")
+    if x.dtype not in _DT and x.dtype != torch.float16:
+        raise TypeError(f"{what} supports float32, bfloat16 and float16 activations, got {x.dtype}")
 
 
 _WS_BYTES = {}
@@ -105,6 +105,12 @@ def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
     lib = _lib.load()
     if not x.is_contiguous():
         x = x.contiguous()
+    if x.dtype == torch.float16:
+        # float16 activations (the reference trainer's default AMP dtype, train.py:180,438; its
+        # fused twin dispatches fp16 too, haar_common.cuh:55-77) are widened at the boundary: the
+        # fp32 kernels run on the exact fp16 values and the result is rounded to fp16 once.
+        out, _ = _forward_impl(x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L)
+        return out.to(torch.float16), x
     pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
     shape = tuple(x.shape)
     with _on_device(x.device):
@@ -126,6 +132,10 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
     base_s, wt_ws[0..L-1], wt_ss[0..L-1] (all None when not needed), in the parameters' dtypes."""
     lib = _lib.load()
     g = grad_out
+    if x.dtype == torch.float16:          # widened at the boundary, as in the forward pass
+        grad_x, grads = _backward_impl(g.float(), x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L,
+                                       need_x, need_params)
+        return (grad_x.to(torch.float16) if grad_x is not None else None), grads
     if g.dtype != x.dtype:
         g = g.to(x.dtype)
     if not g.is_contiguous():
