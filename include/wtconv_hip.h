@@ -88,6 +88,22 @@ int wtconv2d_forward(const void* x, void* out, const wtconv_params* params,
                      int dtype, int param_dtype,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* wtconv2d_forward without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  The scratch that wtconv2d_forward
+ * takes from `workspace` (folded parameters) lives in a static device array of
+ * wtconv_static_scratch_bytes() = 4 MiB that each GPU the library runs on holds until the
+ * process ends; shapes whose forward pass needs more (planes too large for LDS, which stage
+ * a pyramid in the workspace) are rejected with WTCONV_E_UNSUPPORTED.  The call allocates and
+ * frees nothing.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (two streams, two threads) race; calls on one stream are ordered and safe.  The result is
+ * bit-identical to wtconv2d_forward. */
+size_t wtconv_static_scratch_bytes(void);
+
+int wtconv2d_forward_static(const void* x, void* out, const wtconv_params* params,
+                            int B, int C, int H, int W, int K, int levels,
+                            int dtype, int param_dtype, void* stream);
+
 /* grad_x from grad_out: replaces autograd through wtconv2d.py:38-82 and
  * WaveletBranchFunction.backward + conv2d_input (haar_cuda.py:359-413,650-656). */
 int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params,

@@ -31,6 +31,8 @@ EXPORTS = {
 _p, _i, _z = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 for _name in ("wtconv2d_forward", "wtconv2d_backward_input"):
     EXPORTS[_name] = (_i, [_p, _p, ctypes.POINTER(Params)] + [_i] * 8 + [_p, _z, _p])
+EXPORTS["wtconv_static_scratch_bytes"] = (_z, [])
+EXPORTS["wtconv2d_forward_static"] = (_i, [_p, _p, ctypes.POINTER(Params)] + [_i] * 8 + [_p])
 EXPORTS["wtconv2d_backward_params"] = (
     _i, [_p, _p, ctypes.POINTER(Params), ctypes.POINTER(ParamGrads)] + [_i] * 8 + [_p, _z, _p])
 for _name in ("wtconv1d_forward", "wtconv1d_backward_input"):

@@ -657,6 +657,37 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
                              : run_tile1d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
 }
 
+// ---- static scratch for callers that may not allocate ------------------------------------
+// One array per GPU the library runs on, held until the process ends.  Host code never uses the
+// array's name as an address: the device address is looked up once per device and cached.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+constexpr int kMaxDevices = 64;
+#ifndef WT_EMULATE
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(const char* fn, void** ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "%s: hipGetDevice: %s", fn, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(WTCONV_E_UNSUPPORTED, "%s: device index %d", fn, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(WTCONV_E_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+#else
+static unsigned char scratch[kStaticScratchBytes];
+static int static_scratch(const char*, void** ptr) { *ptr = scratch; return 0; }
+#endif
+
 }  // namespace wt
 
 using namespace wt;
@@ -695,6 +726,22 @@ int wtconv2d_forward(const void* x, void* out, const wtconv_params* params, int 
                      void* stream) {
   return plane2d_pass("wtconv2d_forward", x, out, params, B, C, H, W, K, levels, dtype, param_dtype, workspace,
                       workspace_bytes, stream, 0);
+}
+
+size_t wtconv_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int wtconv2d_forward_static(const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
+                            int K, int levels, int dtype, int param_dtype, void* stream) {
+  const char* fn = "wtconv2d_forward_static";
+  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, levels, WTCONV_PASS_FORWARD);
+  if (need > kStaticScratchBytes)
+    return fail(WTCONV_E_UNSUPPORTED,
+                "%s: this shape needs %zu B of scratch, the static buffer holds %zu B; use wtconv2d_forward with a "
+                "caller-supplied workspace", fn, need, kStaticScratchBytes);
+  void* ptr = nullptr;
+  if (int e = static_scratch(fn, &ptr)) return e;
+  return plane2d_pass(fn, x, out, params, B, C, H, W, K, levels, dtype, param_dtype, ptr, kStaticScratchBytes,
+                      stream, 0);
 }
 
 int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_params* params, int B, int C,
