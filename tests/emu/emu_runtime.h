@@ -39,8 +39,10 @@ typedef void* hipStream_t;
 namespace emu {
 struct BlockState {
   std::unique_ptr<std::barrier<>> bar;
+  std::vector<std::unique_ptr<std::barrier<>>> wave_bar;   // one per wavefront of 64 threads
   float* lds = nullptr;
   std::vector<float> xchg;
+  std::vector<uint16_t> mfma_a, mfma_b;                   // [thread][8] operand exchange of the emulated MFMA
   unsigned nthreads = 0;
 };
 inline thread_local BlockState* tls_block = nullptr;
@@ -66,6 +68,31 @@ inline float __shfl_xor(float v, int mask, int /*width*/) {
 }
 
 namespace emu {
+// Barrier over the 64 threads of the calling thread's wavefront.
+inline void wave_barrier() { tls_block->wave_bar[threadIdx.x / 64]->arrive_and_wait(); }
+
+// D = A (16x32) * B (32x16) + C on bfloat16 operands with float accumulation, operands and
+// result distributed over the 64 lanes of a wavefront as v_mfma_f32_16x16x32_bf16 holds them:
+// lane l carries A[l % 16][8 * (l / 16) + j], B[8 * (l / 16) + j][l % 16] (j = 0..7) and
+// D[4 * (l / 16) + r][l % 16] (r = 0..3).  Every lane of the wavefront must call it.
+inline void mfma_16x16x32_bf16(const uint16_t (&a)[8], const uint16_t (&b)[8], float (&c)[4]) {
+  BlockState* st = tls_block;
+  const unsigned t = threadIdx.x, wbase = t / 64 * 64, l = t % 64;
+  for (int j = 0; j < 8; ++j) { st->mfma_a[t * 8 + j] = a[j]; st->mfma_b[t * 8 + j] = b[j]; }
+  wave_barrier();
+  auto f = [](uint16_t v) { uint32_t u = static_cast<uint32_t>(v) << 16; float x; std::memcpy(&x, &u, 4); return x; };
+  const unsigned n = l % 16, q = l / 16;
+  for (int r = 0; r < 4; ++r) {
+    const unsigned m = 4 * q + r;
+    float acc = c[r];
+    for (unsigned kq = 0; kq < 4; ++kq)
+      for (int j = 0; j < 8; ++j)
+        acc += f(st->mfma_a[(wbase + 16 * kq + m) * 8 + j]) * f(st->mfma_b[(wbase + 16 * kq + n) * 8 + j]);
+    c[r] = acc;
+  }
+  wave_barrier();
+}
+
 template <typename F>
 void launch(dim3 grid, dim3 block, size_t lds_bytes, F body) {
   const unsigned nt = block.x * block.y * block.z;
@@ -76,6 +103,12 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, F body) {
         st.bar = std::make_unique<std::barrier<>>(nt);
         st.nthreads = nt;
         st.xchg.assign(nt, 0.f);
+        st.mfma_a.assign(static_cast<size_t>(nt) * 8, 0);
+        st.mfma_b.assign(static_cast<size_t>(nt) * 8, 0);
+        for (unsigned wv = 0; wv < (nt + 63) / 64; ++wv) {
+          const unsigned in_wave = nt - wv * 64 < 64 ? nt - wv * 64 : 64;
+          st.wave_bar.push_back(std::make_unique<std::barrier<>>(in_wave));
+        }
         // exact size: ASan red zones catch LDS overruns; filled with NaN so that reads of
         // never-written LDS show up in results
         float* lds = lds_bytes ? static_cast<float*>(std::aligned_alloc(16, (lds_bytes + 15) / 16 * 16)) : nullptr;

@@ -10,9 +10,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EMU_DIR = os.path.join(ROOT, "tests", "emu")
 BUILD_DIR = os.path.join(EMU_DIR, "_build")
 EXE = os.path.join(BUILD_DIR, "emu_driver")
-SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(EMU_DIR, "emu_driver.cpp")]
+SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(ROOT, "wtconv_amd", "csrc", "mfma2d.hip"),
+           os.path.join(EMU_DIR, "emu_driver.cpp")]
 DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
-                  ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_stream.h", "plan.h")] + [
+                  ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h",
+                   "kernels2d_stream.h", "mfma2d.h", "plan.h")] + [
     os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
 
 
@@ -25,12 +27,13 @@ def build(force=False):
     # -O0 -g1: the run time is dominated by thread creation, the build time by optimisation
     cmd = ["g++", "-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined",
            "-fno-sanitize-recover=undefined", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
-           SOURCES[0], SOURCES[1], "-pthread", "-o", EXE]
+           *SOURCES, "-pthread", "-o", EXE]
     subprocess.run(cmd, check=True, cwd=ROOT)
     return EXE
 
 
-def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600, lds_limit=None):
+def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600, lds_limit=None,
+        mfma=None):
     """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays.
     `lds_limit` (bytes) lowers the LDS budget of the dispatch, so that small planes take the
     level-by-level kernels that real runs only use for planes beyond 160 KB."""
@@ -62,6 +65,9 @@ def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, 
         env.pop("WT_EMU_LDS_LIMIT", None)
         if lds_limit is not None:
             env["WT_EMU_LDS_LIMIT"] = str(int(lds_limit))
+        env.pop("WTCONV_MFMA", None)
+        if mfma is not None:      # 0: vector-ALU kernels only; 1: matrix cores for bf16; 2: for bf16 and fp32
+            env["WTCONV_MFMA"] = str(int(mfma))
         r = subprocess.run([exe, fin, fout], capture_output=True, text=True, timeout=timeout, env=env)
         if r.returncode != 0:
             raise RuntimeError(f"emu_driver failed ({r.returncode}):\n{r.stderr[-4000:]}")

@@ -5,14 +5,17 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libwtconv_hip.so")
-SOURCES = [os.path.join(CSRC, "api.hip")]
-HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_stream.h", "plan.h")] + [
+SOURCES = [os.path.join(CSRC, "api.hip"), os.path.join(CSRC, "mfma2d.hip")]
+HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h",
+                                         "kernels2d_stream.h", "mfma2d.h", "plan.h")] + [
     os.path.join(os.path.dirname(PKG_DIR), "include", "wtconv_hip.h")]
 
 # packed-FP32 code generation is switched off on purpose: every float op is a scalar VALU op
-HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-mllvm", "-amdgpu-mfma-vgpr-form=1",     # MFMA accumulators in ordinary VGPRs: no copies to and from AGPRs
                "-Wno-unused-command-line-argument"]
+OBJ_DIR = os.path.join(PKG_DIR, "build")
 
 
 def hipcc_path():
@@ -23,13 +26,29 @@ def hipcc_path():
 
 
 def build_library(verbose=False):
-    """Compile the HIP sources (always recompiles)."""
-    cmd = [hipcc_path()] + HIPCC_FLAGS + SOURCES + ["-o", LIB_PATH + ".tmp"]
+    """Compile the HIP sources (always recompiles; one hipcc process per source, side by side) and link."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs, procs = [], []
+    for src in SOURCES:
+        obj = os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(src))[0] + ".o")
+        cmd = [hipcc_path()] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        objs.append(obj)
+        procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True))
+    errs = []
+    for pr in procs:
+        so, se = pr.communicate()
+        if pr.returncode != 0:
+            errs.append(so[-4000:] + se[-8000:])
+    if errs:
+        raise RuntimeError("hipcc failed:\n" + "\n".join(errs))
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB_PATH + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + r.stdout[-4000:] + r.stderr[-8000:])
+        raise RuntimeError("link failed:\n" + r.stdout[-4000:] + r.stderr[-8000:])
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     return LIB_PATH
 

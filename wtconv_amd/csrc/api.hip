@@ -1,15 +1,13 @@
 // C ABI of libwtconv_hip.so (declared in include/wtconv_hip.h): argument checks, LDS
 // planning and kernel launches.  Nothing here allocates, frees or synchronises.
-#include <stdarg.h>
-#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
-#include <functional>
 #include <mutex>
-#include <unordered_map>
 
 #include "common.h"
+#include "host_util.h"
+#include "mfma2d.h"
 #include "kernels1d.h"
 #include "kernels1d_row.h"
 #include "kernels2d.h"
@@ -17,121 +15,6 @@
 #include "plan.h"
 
 namespace wt {
-
-static thread_local char g_err[512] = "";
-
-static int fail(int code, const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
-  va_end(ap);
-  return code;
-}
-
-#ifdef WT_EMULATE
-#define WT_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
-  ::emu::launch((grid), (block), (lds_bytes), [&]() { kernel(__VA_ARGS__); })
-static int check_launch(const char*) { return 0; }
-template <typename F> static int allow_lds(F, size_t) { return 0; }
-#else
-#define WT_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
-  hipLaunchKernelGGL(kernel, (grid), (block), (lds_bytes), (stream), __VA_ARGS__)
-static int check_launch(const char* what) {
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
-  return 0;
-}
-// Per-kernel facts that cost a driver call (hundreds of nanoseconds to microseconds each) are
-// looked up once per (device, kernel, launch shape) and kept for the life of the process.
-struct KernelKey {
-  int dev; const void* fn; int block; size_t lds;
-  bool operator==(const KernelKey& o) const { return dev == o.dev && fn == o.fn && block == o.block && lds == o.lds; }
-};
-struct KernelKeyHash {
-  size_t operator()(const KernelKey& k) const {
-    return std::hash<const void*>()(k.fn) ^ (static_cast<size_t>(k.dev) * 0x9e3779b97f4a7c15ull) ^
-           (k.lds * 31 + static_cast<size_t>(k.block));
-  }
-};
-static std::mutex g_kernel_cache_mutex;
-static std::unordered_map<KernelKey, int, KernelKeyHash> g_lds_allowed, g_resident;
-
-static int current_device() {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); dev = 0; }
-  return dev;
-}
-
-// Workgroups above 64 KiB of dynamic LDS need the opt-in attribute (set once per kernel and size).
-template <typename F> static int allow_lds(F kernel, size_t bytes) {
-  if (bytes <= 64 * 1024) return 0;
-  const KernelKey key = {current_device(), reinterpret_cast<const void*>(kernel), 0, bytes};
-  {
-    std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
-    if (g_lds_allowed.count(key)) return 0;
-  }
-  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(bytes));
-  if (e != hipSuccess) return fail(WTCONV_E_LAUNCH, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
-  std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
-  g_lds_allowed[key] = 1;
-  return 0;
-}
-#endif
-
-// Compute units of the current device (cached per thread; 256 on MI355X).
-static int compute_units() {
-#ifdef WT_EMULATE
-  return 2;
-#else
-  static thread_local int cached_dev = -1, cached_cu = 0;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 256;
-  if (dev != cached_dev) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached_dev = dev;
-    cached_cu = n;
-  }
-  return cached_cu;
-#endif
-}
-
-// Workgroups of `kernel` that fit on one CU at once (registers, LDS, wave slots): the grid
-// of a persistent kernel must not exceed CUs x this, or the surplus runs as a second round.
-template <typename F>
-static int resident_per_cu(F kernel, int block, size_t lds_bytes) {
-#ifdef WT_EMULATE
-  (void)kernel; (void)block; (void)lds_bytes;
-  return 1;
-#else
-  const KernelKey key = {current_device(), reinterpret_cast<const void*>(kernel), block, lds_bytes};
-  {
-    std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
-    auto it = g_resident.find(key);
-    if (it != g_resident.end()) return it->second;
-  }
-  int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kernel), block, lds_bytes) !=
-          hipSuccess || n < 1) {
-    (void)hipGetLastError();
-    n = resident_workgroups(1, lds_bytes, block / 64, 8);
-  }
-  std::lock_guard<std::mutex> lock(g_kernel_cache_mutex);
-  g_resident[key] = n;
-  return n;
-#endif
-}
-
-static ParamTable to_table(const wtconv_params* p, int L) {
-  ParamTable t = {};
-  t.base_weight = p->base_weight;
-  t.base_bias = p->base_bias;
-  t.base_scale = p->base_scale;
-  for (int l = 0; l < L; ++l) { t.wt_weight[l] = p->wt_weight[l]; t.wt_scale[l] = p->wt_scale[l]; }
-  return t;
-}
 
 static int check_common(const char* fn, const wtconv_params* params, int B, int C, int K, int L,
                         int dtype, int pdtype) {
@@ -435,6 +318,8 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
   if (static_cast<long long>(B) * C > 0x7fffffffLL / 4)
     return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld is too large", fn, static_cast<long long>(B) * C);
+  if (mfma2d_query(B, C, H, W, K, L, dtype).ok)
+    return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, ws, ws_bytes, stream, flip);
   if (!plane_fits_lds(B, C, H, W, K, L)) {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     float* fw = static_cast<float*>(ws);
@@ -715,8 +600,16 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
                2 * make_stream2d(B, C, H, W, levels).floats;
     }
   } else {
+    // the dtype is not an argument here: size for the larger of the two (fp32 tensors take
+    // three split tables) whenever either could run on the matrix-core kernels
+    size_t mf = 0;
+    for (int dt : {WTCONV_F32, WTCONV_BF16}) {
+      const Mfma2dQuery q = mfma2d_query(B, C, H, W, K, levels, dt);
+      if (q.ok && q.ws_bytes > mf) mf = q.ws_bytes;
+    }
     floats = fold_floats(C, 4, levels, K * K);
     if (!plane_fits_lds(B, C, H, W, K, levels)) floats = round_up64(floats) + make_stream2d(B, C, H, W, levels).floats;
+    if (mf > floats * sizeof(float)) floats = (mf + 3) / 4;
   }
   return (floats * sizeof(float) + 255) / 256 * 256;
 }

@@ -1,0 +1,207 @@
+// Host side of the matrix-core 2-D path: LDS planning, dispatch and launches of
+// kernels2d_mfma.h.  Allocates nothing, never synchronises.
+#include <stdlib.h>
+#include <string.h>
+
+#include "common.h"
+#include "host_util.h"
+#include "kernels2d_mfma.h"
+#include "mfma2d.h"
+
+namespace wt {
+
+namespace {
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// LDS layout and unit geometry for `pb` planes per unit; false if the kernel cannot index it.
+bool make_mplan(int B, int C, int H, int W, int L, int NS, int pb, MPlan* out) {
+  if (!make_mplan_geometry(H, W, L, NS, pb, out)) return false;
+  out->B = B; out->C = C;
+  out->upc = ceil_div(B, pb);
+  if (static_cast<long long>(C) * out->upc > 0x7fffffffLL) return false;
+  out->nunits = C * out->upc;
+  if (static_cast<long long>(pb) * C * H * W > 0x7fffffffLL) return false;
+  return true;
+}
+
+// Which tensors take the matrix-core kernels (environment variable WTCONV_MFMA, read once):
+// 0 none; 1 bf16 tensors (the default); 2 bf16 and fp32 tensors, the latter split into three bf16
+// planes -- exact to fp32 rounding, but slower than the vector-ALU kernels on the shapes measured.
+int mfma_mode() {
+  static const int mode = [] {
+    const char* e = getenv("WTCONV_MFMA");
+    return e ? atoi(e) : 1;
+  }();
+  return mode;
+}
+
+size_t lds_budget() {
+#ifdef WT_EMULATE
+  if (const char* e = getenv("WT_EMU_LDS_LIMIT")) return static_cast<size_t>(atol(e));
+#endif
+  return kLdsLimitBytes;
+}
+
+// Planes per unit: as many as keep every thread's share at one 4x4 block, shrunk until a
+// workgroup's LDS leaves room for several workgroups per CU.
+bool choose_mplan_uncached(int B, int C, int H, int W, int L, int NS, MPlan* out, int* nbl);
+
+// Plans are pure functions of the shape; the search behind them (candidate plane counts, checked
+// reciprocals) is too slow to repeat on every call, so results are kept per thread.
+struct PlanKey {
+  int B, C, H, W, L, NS;
+  bool operator==(const PlanKey& o) const { return B == o.B && C == o.C && H == o.H && W == o.W && L == o.L && NS == o.NS; }
+};
+struct PlanKeyHash {
+  size_t operator()(const PlanKey& k) const {
+    size_t h = 1469598103934665603ull;
+    for (int v : {k.B, k.C, k.H, k.W, k.L, k.NS}) h = (h ^ static_cast<size_t>(v)) * 1099511628211ull;
+    return h;
+  }
+};
+struct PlanVal { bool ok; MPlan pl; int nbl; };
+
+bool choose_mplan(int B, int C, int H, int W, int L, int NS, MPlan* out, int* nbl) {
+  static thread_local std::unordered_map<PlanKey, PlanVal, PlanKeyHash> cache;
+  const PlanKey key = {B, C, H, W, L, NS};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    if (cache.size() > 4096) cache.clear();
+    PlanVal v = {};
+    v.ok = choose_mplan_uncached(B, C, H, W, L, NS, &v.pl, &v.nbl);
+    it = cache.emplace(key, v).first;
+  }
+  if (it->second.ok) { *out = it->second.pl; *nbl = it->second.nbl; }
+  return it->second.ok;
+}
+
+bool choose_mplan_uncached(int B, int C, int H, int W, int L, int NS, MPlan* out, int* nbl) {
+  const int bpp0 = ceil_div(H, 4) * ceil_div(W, 4);
+  int pb = kMfmaBlock / bpp0;
+  if (pb < 1) pb = 1;
+  if (pb > B) pb = B;
+  // Four workgroups per CU (40 KB each) where the planes allow it; three (53 KB) if that puts
+  // clearly more threads to work in the load phase of planes of 14 x 14 and larger (measured, bf16,
+  // stage shapes: 28 x 28 planes 48 -> 44 us with 4 instead of 3 planes; 7 x 7 planes are faster
+  // with 27 planes and four workgroups than with 32 and three).
+  const size_t want = NS == 1 ? 40 * 1024 : 80 * 1024, relaxed = NS == 1 ? 53 * 1024 : 80 * 1024;
+  const int pb_max = pb;
+  MPlan pl;
+  for (;; --pb) {
+    if (!make_mplan(B, C, H, W, L, NS, pb, &pl)) return false;
+    if (static_cast<size_t>(pl.lds_bytes) <= want || pb == 1) break;
+  }
+  if (bpp0 >= 16 && pl.nblk[0] * 10 < kMfmaBlock * 6) {
+    for (int p2 = pb_max; p2 > pb; --p2) {
+      MPlan alt;
+      if (B % p2 == 0 && make_mplan(B, C, H, W, L, NS, p2, &alt) && static_cast<size_t>(alt.lds_bytes) <= relaxed) {
+        pl = alt;
+        pb = p2;
+        break;
+      }
+    }
+  }
+  if (static_cast<size_t>(pl.lds_bytes) > lds_budget()) return false;
+  const int per_thread = ceil_div(pl.nblk[0], kMfmaBlock);
+  if (per_thread > 4) return false;
+  *nbl = per_thread <= 1 ? 1 : (per_thread == 2 ? 2 : 4);
+  *out = pl;
+  return true;
+}
+
+size_t table_bytes(int C, int L, int NS) {
+  return (static_cast<size_t>(C) * NS * (1 + 4 * L) * kFragEntries * 16 + 255) / 256 * 256;
+}
+
+template <typename T, int NS, int NBL, bool VEC, typename Geo>
+int launch_mfma(const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl, hipStream_t stream) {
+  auto kern = wt2d_mfma_kernel<T, NS, NBL, VEC, NS == 1, Geo>;
+  const size_t lds = static_cast<size_t>(pl.lds_bytes);
+  if (int e = allow_lds(kern, lds)) return e;
+  int nwg = compute_units() * resident_per_cu(kern, kMfmaBlock, lds);
+  if (nwg > pl.nunits) nwg = pl.nunits;
+  WT_LAUNCH(kern, dim3(nwg), dim3(kMfmaBlock), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), tg, fb, pl);
+  return check_launch("wt2d_mfma_kernel");
+}
+
+template <typename T, int NS, int NBL>
+int launch_mfma_vec(bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+                    hipStream_t stream) {
+  return vec ? launch_mfma<T, NS, NBL, true, GeoRuntime>(x, out, tg, fb, pl, stream)
+             : launch_mfma<T, NS, NBL, false, GeoRuntime>(x, out, tg, fb, pl, stream);
+}
+
+// The WTConvNeXt stage shapes (56/28/14/7 squares; 3/3/2/2 levels as single layers, 5/4/3/2 in the
+// model) have kernels whose whole LDS layout is a compile-time constant.
+template <typename T, int NS, int H, int L, int PB, bool VEC>
+bool try_static(bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+                hipStream_t stream, int* rc) {
+  if (pl.H != H || pl.W != H || pl.L != L || pl.pb != PB || vec != VEC) return false;
+  *rc = launch_mfma<T, NS, 1, VEC, GeoStatic<H, H, L, PB>>(x, out, tg, fb, pl, stream);
+  return true;
+}
+
+template <typename T, int NS>
+int launch_mfma_nbl(int nbl, bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+                    hipStream_t stream) {
+#ifndef WT_EMULATE
+  int rc = 0;
+#define WT_TRY(H_, L_, PB_, VEC_) \
+  if (try_static<T, NS, H_, L_, PB_, VEC_>(vec, x, out, tg, fb, pl, stream, &rc)) return rc;
+  if constexpr (NS == 1) {
+    WT_TRY(56, 3, 1, true) WT_TRY(28, 3, 4, true) WT_TRY(14, 2, 11, false) WT_TRY(7, 2, 29, false)
+    WT_TRY(56, 5, 1, true) WT_TRY(28, 4, 4, true) WT_TRY(14, 3, 9, false)
+  }
+#undef WT_TRY
+#endif
+  switch (nbl) {
+    case 1: return launch_mfma_vec<T, NS, 1>(vec, x, out, tg, fb, pl, stream);
+    case 2: return launch_mfma_vec<T, NS, 2>(vec, x, out, tg, fb, pl, stream);
+    default: return launch_mfma_vec<T, NS, 4>(vec, x, out, tg, fb, pl, stream);
+  }
+}
+
+}  // namespace
+
+Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype) {
+  Mfma2dQuery r = {false, 0};
+  const int mode = mfma_mode();
+  if (mode <= 0 || K > 5 || L < 1 || L > kMaxLevels) return r;
+  if (dtype == WTCONV_F32 && mode < 2) return r;
+  const int NS = dtype == WTCONV_F32 ? 3 : 1;
+  MPlan pl;
+  int nbl;
+  if (!choose_mplan(B, C, H, W, L, NS, &pl, &nbl)) return r;
+  r.ok = true;
+  r.ws_bytes = table_bytes(C, L, NS) + (static_cast<size_t>(C) * sizeof(float) + 255) / 256 * 256;
+  return r;
+}
+
+int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
+                int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes, hipStream_t stream, int flip) {
+  const int NS = dtype == WTCONV_F32 ? 3 : 1;
+  MPlan pl;
+  int nbl;
+  if (!choose_mplan(B, C, H, W, L, NS, &pl, &nbl))
+    return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
+  const size_t tb = table_bytes(C, L, NS);
+  if (ws == nullptr || ws_bytes < tb + static_cast<size_t>(C) * sizeof(float))
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace too small for the fragment tables", fn);
+  uint4* tg = static_cast<uint4*>(ws);
+  float* fb = reinterpret_cast<float*>(static_cast<char*>(ws) + tb);
+  const int total = C * pl.nfilt * kFragEntries;
+  int blocks = (total + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  WT_LAUNCH(fold_frag_kernel, dim3(blocks), dim3(256), 0, stream, to_table(params, L), pdtype, tg, fb, C, L, K, NS,
+            flip, flip ? 0 : 1);
+  if (int e = check_launch("fold_frag_kernel")) return e;
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  const uintptr_t mask = 4 * esz - 1;
+  const bool vec = (W % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & mask) == 0 &&
+                   (reinterpret_cast<uintptr_t>(out) & mask) == 0;
+  return dtype == WTCONV_F32 ? launch_mfma_nbl<float, 3>(nbl, vec, x, out, tg, fb, pl, stream)
+                             : launch_mfma_nbl<bf16_t, 1>(nbl, vec, x, out, tg, fb, pl, stream);
+}
+
+}  // namespace wt

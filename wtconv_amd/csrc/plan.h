@@ -4,6 +4,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "host_util.h"
 #include "kernels1d.h"
 #include "kernels2d.h"
 
@@ -143,30 +144,6 @@ inline void finish_wgrad_plan(Plan2D* pl, int K) {
     pl->prefetch = nps / gs >= pl->h[1];       // one 2x4 piece per thread covers the plane
     if (pl->prefetch && pl->pb == 1 && gs <= 16 && pl->L >= 2) pl->fuse = pl->L >= 3 ? 3 : 2;
   }
-}
-
-// Batch chunking of the 2-D weight-gradient kernel; a chunk is a whole number of
-// iterations of `pb` planes.  `resident` = workgroups the device holds at once.
-inline void wgrad_chunks(int B, int C, int pb, int resident, int* bchunk, int* nchunk) {
-  // Chunks per channel n: C*n workgroups run in ceil(C*n/resident) rounds.  Every workgroup
-  // pays LDS zeroing, a cold first fetch and the final reduction once, so score = fill of
-  // the rounds minus 9 % per round, and the best n wins (ties: the smaller).  The penalty is
-  // fitted to measurements (us per launch): 192 channels of 28x28 run best as 5 chunks (2 rounds,
-  // 154) rather than 8 (3 full rounds, 168) or 2 (1 round three-quarters full, 177); 384
-  // channels of 14x14 as 4 (131; 1 chunk: 145); 768 channels of 7x7 as 2; 96 channels of 56x56 as 5.
-  const int iters = (B + pb - 1) / pb;           // iterations available per channel
-  int best_n = 1;
-  double best = -1.0;
-  for (int n = 1; n <= iters && n <= 64; ++n) {
-    const int wgs = C * n;
-    const int rounds = (wgs + resident - 1) / resident;
-    const double score = static_cast<double>(wgs) / (static_cast<double>(rounds) * resident) - 0.09 * rounds;
-    if (score > best + 1e-9) { best = score; best_n = n; }
-  }
-  int bc = (iters + best_n - 1) / best_n * pb;
-  if (bc < 1) bc = 1;
-  *bchunk = bc;
-  *nchunk = (B + bc - 1) / bc;
 }
 
 // ---- 1-D ------------------------------------------------------------------------------
