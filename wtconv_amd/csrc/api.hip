@@ -319,7 +319,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   if (static_cast<long long>(B) * C > 0x7fffffffLL / 4)
     return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld is too large", fn, static_cast<long long>(B) * C);
   if (mfma2d_query(B, C, H, W, K, L, dtype).ok)
-    return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, ws, ws_bytes, stream, flip);
+    return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, stream, flip);
   if (!plane_fits_lds(B, C, H, W, K, L)) {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     float* fw = static_cast<float*>(ws);

@@ -118,7 +118,10 @@ constexpr bool make_mplan_geometry(int H, int W, int L, int NS, int pb, MPlan* o
     pl.zpitch[l] = 4 * pl.nbc[l - 1];
     pl.zpl[l] = 4 * pl.nbr[l - 1] * pl.zpitch[l];
     pl.zoff[l] = off;
-    off += pb * pl.zpl[l] * 4;
+    int zbytes = pb * pl.zpl[l] * 4;
+    const int staging = NS * pl.tfirst * kFragEntries * 16;      // Z_1 doubles as staging area when a channel's parameters are folded
+    if (l == 1 && zbytes < staging) zbytes = staging;
+    off += zbytes;
     if (off > (1 << 20)) return false;
   }
   for (int l = 2; l < L; ++l) {
@@ -259,64 +262,54 @@ __device__ __forceinline__ void split_pair(float lo, float hi, uint32_t (&w)[NS]
 }
 
 // ------------------------------------------------------------------ fragment table (fold)
-// tg[((c * NS + j) * nfilt + f) * 21 + e]: split j of filter f of channel c; entry e = 4 kh + cs
-// holds kernel row kh of the filter (embedded in 5 x 5, scaled by gamma and 4^-level, rotated
-// by 180 degrees when flip != 0) shifted right by cs in a window of 8; entry 20 is zero.
-// fb[c] = gamma_b * bias (0 without bias or when use_bias == 0).
-__global__ void fold_frag_kernel(ParamTable p, int pdtype, uint4* __restrict__ tg, float* __restrict__ fb, int C,
-                                 int L, int K, int NS, int flip, int use_bias) {
-  const int nfilt = 1 + 4 * L;
-  const int total = C * nfilt * kFragEntries;
+// Entry e = 4 kh + cs of filter f of channel c: kernel row kh of the filter (embedded in 5 x 5,
+// scaled by gamma and 4^-level, rotated by 180 degrees when flip != 0) shifted right by cs in a
+// window of 8 -- the 8 bf16 a lane feeds the MFMA with -- as NS split words; entry 20 is zero.
+// Filter 0 is the base conv, filter 1 + 4 (l - 1) + s sub-band s of level l.
+template <int NS>
+__device__ __forceinline__ void fold_entry(const ParamTable& p, int pdtype, int K, int flip, int c, int f, int e,
+                                           uint4 (&out)[NS]) {
   const int KK = K * K, o = 2 - K / 2;
-  for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
-    const int e = idx % kFragEntries;
-    const int f = (idx / kFragEntries) % nfilt;
-    const int c = idx / (kFragEntries * nfilt);
-    float v[8];
+  float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = 0.f;
-    if (e < 20) {
-      const int kh = e >> 2, cs = e & 3;
-      const int ih = kh - o;
-      float scale;
-      const void* wp;
-      int ch;
-      if (f == 0) {
-        wp = p.base_weight; ch = c;
-        scale = load_param(p.base_scale, pdtype, c);
-      } else {
-        const int l = (f - 1) >> 2, s = (f - 1) & 3;
-        wp = p.wt_weight[l]; ch = c * 4 + s;
-        scale = load_param(p.wt_scale[l], pdtype, ch);
+  for (int j = 0; j < 8; ++j) v[j] = 0.f;
+  if (e < 20) {
+    const int kh = e >> 2, cs = e & 3;
+    const int ih = kh - o;
+    float scale;
+    const void* wp;
+    int ch;
+    if (f == 0) {
+      wp = p.base_weight; ch = c;
+      scale = load_param(p.base_scale, pdtype, c);
+    } else {
+      const int l = (f - 1) >> 2, s = (f - 1) & 3;
+      wp = p.wt_weight[l]; ch = c * 4 + s;
+      scale = load_param(p.wt_scale[l], pdtype, ch);
 #pragma unroll 1
-        for (int i = 0; i <= l; ++i) scale *= 0.25f;
-      }
-      if (ih >= 0 && ih < K) {
+      for (int i = 0; i <= l; ++i) scale *= 0.25f;
+    }
+    if (ih >= 0 && ih < K) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int iw = j - cs - o;
-          if (iw >= 0 && iw < K && j - cs < 5 && j - cs >= 0) {
-            const int t = ih * K + iw;
-            v[j] = load_param(wp, pdtype, ch * KK + (flip ? KK - 1 - t : t)) * scale;
-          }
+      for (int j = 0; j < 8; ++j) {
+        const int iw = j - cs - o;
+        if (iw >= 0 && iw < K && j - cs < 5 && j - cs >= 0) {
+          const int t = ih * K + iw;
+          v[j] = load_param(wp, pdtype, ch * KK + (flip ? KK - 1 - t : t)) * scale;
         }
       }
     }
-    for (int js = 0; js < NS; ++js) {
-      uint32_t w[4];
+  }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-        v[2 * i] -= __uint_as_float(w[i] << 16);
-        v[2 * i + 1] -= __uint_as_float(w[i] & 0xffff0000u);
-      }
-      uint4 q; q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3];
-      tg[(static_cast<size_t>(c) * NS + js) * nfilt * kFragEntries + f * kFragEntries + e] = q;
+  for (int js = 0; js < NS; ++js) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+      v[2 * i] -= __uint_as_float(w[i] << 16);
+      v[2 * i + 1] -= __uint_as_float(w[i] & 0xffff0000u);
     }
-    if (f == 0 && e == 0)
-      fb[c] = (use_bias && p.base_bias != nullptr)
-                  ? load_param(p.base_bias, pdtype, c) * load_param(p.base_scale, pdtype, c)
-                  : 0.f;
+    out[js].x = w[0]; out[js].y = w[1]; out[js].z = w[2]; out[js].w = w[3];
   }
 }
 
@@ -420,8 +413,8 @@ __device__ __forceinline__ TileLane tile_lane(const char* lds, int T, int n, int
 // in registers while the channel does not change.
 template <typename T, int NS, int NBL, bool VEC, bool RES, typename Geo>
 __global__ void __launch_bounds__(kMfmaBlock, NS == 1 ? 4 : 2)      // waves per SIMD the register budget must allow
-wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const uint4* __restrict__ tg,
-                 const float* __restrict__ fb, const MPlan plarg) {
+wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable prm, int pdtype, int K, int flip,
+                 int use_bias, const MPlan plarg) {
   // the plan: shape-dependent fields from the compile-time constant where there is one
   const MPlan pl = [&]() {
     if constexpr (Geo::kStatic) {
@@ -538,23 +531,32 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const uint4* __re
     const int b0 = (u - c * upc) * pb;
     const int np = B - b0 < pb ? B - b0 : pb;      // planes of this unit that exist
     if (c != cur_c) {     // (the previous unit ended with a barrier: nobody still reads the old table)
-      const int nf_all = pl.nfilt * kFragEntries, nf_lds = (pl.nfilt - pl.tfirst) * kFragEntries;
-      const uint4* src = tg + static_cast<size_t>(c) * NS * nf_all;
+      // fold this channel's parameters into the fragment table: filters from `tfirst` on into their
+      // LDS table, the ones before it (held in registers) through the idle Z_1 buffer
+      const int nent = pl.nfilt * kFragEntries;
+      const int nf_lds = (pl.nfilt - pl.tfirst) * kFragEntries;
+      for (int i = tid; i < nent; i += kMfmaBlock) {
+        const int f = i / kFragEntries, e = i - f * kFragEntries;
+        uint4 w[NS];
+        fold_entry<NS>(prm, pdtype, K, flip, c, f, e, w);
 #pragma unroll
-      for (int j = 0; j < NS; ++j)
-        for (int i = tid; i < nf_lds; i += kMfmaBlock)
-          lds_st<uint4>(lds, toff + (j * nf_lds + i) * 16, src[j * nf_all + pl.tfirst * kFragEntries + i]);
-      bias = fb[c];
+        for (int j = 0; j < NS; ++j) {
+          const int o = f >= pl.tfirst ? toff + (j * nf_lds + i - pl.tfirst * kFragEntries) * 16 : zoff1 + (j * pl.tfirst * kFragEntries + i) * 16;
+          lds_st<uint4>(lds, o, w[j]);
+        }
+      }
+      bias = (use_bias && prm.base_bias != nullptr)
+                 ? load_param(prm.base_bias, pdtype, c) * load_param(prm.base_scale, pdtype, c) : 0.f;
       cur_c = c;
-      if constexpr (RES) {      // base conv and level 1: this lane's fragments straight from the table in HBM (L2)
-        auto gfrag = [&](int f, int ent) {
-          const uint4 v = src[f * kFragEntries + ent];
-          Frag fr; fr.d[0] = v.x; fr.d[1] = v.y; fr.d[2] = v.z; fr.d[3] = v.w;
-          return fr;
-        };
-        ra0t[0] = gfrag(0, ent_top); ra0b[0] = gfrag(0, ent_bot);
+      if constexpr (RES) {
+        WT_LDS_BARRIER();
+        ra0t[0] = lds_frag16(lds, zoff1 + ent_top * 16);
+        ra0b[0] = lds_frag16(lds, zoff1 + ent_bot * 16);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) { ra1t[s][0] = gfrag(1 + s, ent_top); ra1b[s][0] = gfrag(1 + s, ent_bot); }
+        for (int s = 0; s < 4; ++s) {
+          ra1t[s][0] = lds_frag16(lds, zoff1 + ((1 + s) * kFragEntries + ent_top) * 16);
+          ra1b[s][0] = lds_frag16(lds, zoff1 + ((1 + s) * kFragEntries + ent_bot) * 16);
+        }
       }
     }
 

@@ -8,7 +8,7 @@
 namespace wt {
 
 // Whether a forward / input-gradient pass of this shape runs on the MFMA kernels, and the
-// workspace it then needs (fragment tables of every channel + folded bias).
+// workspace it then needs (none: the kernel folds the parameters of a channel itself).
 struct Mfma2dQuery {
   bool ok;
   size_t ws_bytes;
@@ -18,6 +18,6 @@ Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype);
 // One pass (flip = 0: forward, 1: input gradient).  Returns 0 or a WTCONV_E_* code with the
 // message left in the thread's error buffer.
 int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
-                int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes, hipStream_t stream, int flip);
+                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip);
 
 }  // namespace wt

@@ -110,55 +110,60 @@ bool choose_mplan_uncached(int B, int C, int H, int W, int L, int NS, MPlan* out
   return true;
 }
 
-size_t table_bytes(int C, int L, int NS) {
-  return (static_cast<size_t>(C) * NS * (1 + 4 * L) * kFragEntries * 16 + 255) / 256 * 256;
-}
+// Parameter table and folding options of a pass.
+struct MfmaArgs {
+  ParamTable prm;
+  int pdtype, K, flip, use_bias;
+};
 
 template <typename T, int NS, int NBL, bool VEC, typename Geo>
-int launch_mfma(const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl, hipStream_t stream) {
+int launch_mfma(const void* x, void* out, const MfmaArgs& a, const MPlan& pl, hipStream_t stream) {
   auto kern = wt2d_mfma_kernel<T, NS, NBL, VEC, NS == 1, Geo>;
   const size_t lds = static_cast<size_t>(pl.lds_bytes);
   if (int e = allow_lds(kern, lds)) return e;
   int nwg = compute_units() * resident_per_cu(kern, kMfmaBlock, lds);
   if (nwg > pl.nunits) nwg = pl.nunits;
-  WT_LAUNCH(kern, dim3(nwg), dim3(kMfmaBlock), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), tg, fb, pl);
+  WT_LAUNCH(kern, dim3(nwg), dim3(kMfmaBlock), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), a.prm,
+            a.pdtype, a.K, a.flip, a.use_bias, pl);
   return check_launch("wt2d_mfma_kernel");
 }
 
 template <typename T, int NS, int NBL>
-int launch_mfma_vec(bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+int launch_mfma_vec(bool vec, const void* x, void* out, const MfmaArgs& a, const MPlan& pl,
                     hipStream_t stream) {
-  return vec ? launch_mfma<T, NS, NBL, true, GeoRuntime>(x, out, tg, fb, pl, stream)
-             : launch_mfma<T, NS, NBL, false, GeoRuntime>(x, out, tg, fb, pl, stream);
+  return vec ? launch_mfma<T, NS, NBL, true, GeoRuntime>(x, out, a, pl, stream)
+             : launch_mfma<T, NS, NBL, false, GeoRuntime>(x, out, a, pl, stream);
 }
 
 // The WTConvNeXt stage shapes (56/28/14/7 squares; 3/3/2/2 levels as single layers, 5/4/3/2 in the
 // model) have kernels whose whole LDS layout is a compile-time constant.
 template <typename T, int NS, int H, int L, int PB, bool VEC>
-bool try_static(bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+bool try_static(bool vec, const void* x, void* out, const MfmaArgs& a, const MPlan& pl,
                 hipStream_t stream, int* rc) {
   if (pl.H != H || pl.W != H || pl.L != L || pl.pb != PB || vec != VEC) return false;
-  *rc = launch_mfma<T, NS, 1, VEC, GeoStatic<H, H, L, PB>>(x, out, tg, fb, pl, stream);
+  *rc = launch_mfma<T, NS, 1, VEC, GeoStatic<H, H, L, PB>>(x, out, a, pl, stream);
   return true;
 }
 
 template <typename T, int NS>
-int launch_mfma_nbl(int nbl, bool vec, const void* x, void* out, const uint4* tg, const float* fb, const MPlan& pl,
+int launch_mfma_nbl(int nbl, bool vec, const void* x, void* out, const MfmaArgs& a, const MPlan& pl,
                     hipStream_t stream) {
 #ifndef WT_EMULATE
   int rc = 0;
 #define WT_TRY(H_, L_, PB_, VEC_) \
-  if (try_static<T, NS, H_, L_, PB_, VEC_>(vec, x, out, tg, fb, pl, stream, &rc)) return rc;
+  if (try_static<T, NS, H_, L_, PB_, VEC_>(vec, x, out, a, pl, stream, &rc)) return rc;
   if constexpr (NS == 1) {
     WT_TRY(56, 3, 1, true) WT_TRY(28, 3, 4, true) WT_TRY(14, 2, 11, false) WT_TRY(7, 2, 29, false)
     WT_TRY(56, 5, 1, true) WT_TRY(28, 4, 4, true) WT_TRY(14, 3, 9, false)
+  } else {
+    WT_TRY(56, 3, 1, true) WT_TRY(28, 3, 2, true) WT_TRY(14, 2, 9, false) WT_TRY(7, 2, 21, false)
   }
 #undef WT_TRY
 #endif
   switch (nbl) {
-    case 1: return launch_mfma_vec<T, NS, 1>(vec, x, out, tg, fb, pl, stream);
-    case 2: return launch_mfma_vec<T, NS, 2>(vec, x, out, tg, fb, pl, stream);
-    default: return launch_mfma_vec<T, NS, 4>(vec, x, out, tg, fb, pl, stream);
+    case 1: return launch_mfma_vec<T, NS, 1>(vec, x, out, a, pl, stream);
+    case 2: return launch_mfma_vec<T, NS, 2>(vec, x, out, a, pl, stream);
+    default: return launch_mfma_vec<T, NS, 4>(vec, x, out, a, pl, stream);
   }
 }
 
@@ -174,34 +179,24 @@ Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype) {
   int nbl;
   if (!choose_mplan(B, C, H, W, L, NS, &pl, &nbl)) return r;
   r.ok = true;
-  r.ws_bytes = table_bytes(C, L, NS) + (static_cast<size_t>(C) * sizeof(float) + 255) / 256 * 256;
+  r.ws_bytes = 0;       // the kernel folds the parameters of a channel itself
   return r;
 }
 
 int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
-                int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes, hipStream_t stream, int flip) {
+                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip) {
   const int NS = dtype == WTCONV_F32 ? 3 : 1;
   MPlan pl;
   int nbl;
   if (!choose_mplan(B, C, H, W, L, NS, &pl, &nbl))
     return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
-  const size_t tb = table_bytes(C, L, NS);
-  if (ws == nullptr || ws_bytes < tb + static_cast<size_t>(C) * sizeof(float))
-    return fail(WTCONV_E_WORKSPACE, "%s: workspace too small for the fragment tables", fn);
-  uint4* tg = static_cast<uint4*>(ws);
-  float* fb = reinterpret_cast<float*>(static_cast<char*>(ws) + tb);
-  const int total = C * pl.nfilt * kFragEntries;
-  int blocks = (total + 255) / 256;
-  if (blocks > 2048) blocks = 2048;
-  WT_LAUNCH(fold_frag_kernel, dim3(blocks), dim3(256), 0, stream, to_table(params, L), pdtype, tg, fb, C, L, K, NS,
-            flip, flip ? 0 : 1);
-  if (int e = check_launch("fold_frag_kernel")) return e;
+  const MfmaArgs a = {to_table(params, L), pdtype, K, flip, flip ? 0 : 1};
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   const uintptr_t mask = 4 * esz - 1;
   const bool vec = (W % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & mask) == 0 &&
                    (reinterpret_cast<uintptr_t>(out) & mask) == 0;
-  return dtype == WTCONV_F32 ? launch_mfma_nbl<float, 3>(nbl, vec, x, out, tg, fb, pl, stream)
-                             : launch_mfma_nbl<bf16_t, 1>(nbl, vec, x, out, tg, fb, pl, stream);
+  return dtype == WTCONV_F32 ? launch_mfma_nbl<float, 3>(nbl, vec, x, out, a, pl, stream)
+                             : launch_mfma_nbl<bf16_t, 1>(nbl, vec, x, out, a, pl, stream);
 }
 
 }  // namespace wt
