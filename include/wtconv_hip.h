@@ -26,7 +26,7 @@ extern "C" {
 #endif
 
 #define WTCONV_MAX_LEVELS 5
-#define WTCONV_ABI_VERSION 1
+#define WTCONV_ABI_VERSION 2
 
 enum { WTCONV_F32 = 0, WTCONV_BF16 = 1 };
 
@@ -38,7 +38,10 @@ enum {
   WTCONV_E_LAUNCH = -4      /* HIP reported a launch error                           */
 };
 
-enum { WTCONV_PASS_FORWARD = 0, WTCONV_PASS_BACKWARD_INPUT = 1, WTCONV_PASS_BACKWARD_PARAMS = 2 };
+enum {
+  WTCONV_PASS_FORWARD = 0, WTCONV_PASS_BACKWARD_INPUT = 1, WTCONV_PASS_BACKWARD_PARAMS = 2,
+  WTCONV_PASS_BACKWARD = 3   /* wtconv*_backward: input and parameter gradients in one call */
+};
 
 /* Device pointers to the layer's parameters, in the reference module's own tensor
  * layouts (wtconv/wtconv2d.py:23-31, wtconv/wtconv1d.py:23-31):
@@ -120,6 +123,17 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
                              int dtype, int param_dtype,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* The whole backward pass in one call: grad_x and every parameter gradient, as
+ * WaveletBranchFunction.backward + ScaledDepthwiseConvFunction.backward produce them in one
+ * autograd node each (haar_cuda.py:359-424,650-676).  Same as wtconv2d_backward_input followed
+ * by wtconv2d_backward_params on `stream`, sharing `workspace`
+ * (wtconv2d_workspace_bytes(..., WTCONV_PASS_BACKWARD) bytes). */
+int wtconv2d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
+                      const wtconv_param_grads* grads,
+                      int B, int C, int H, int W, int K, int levels,
+                      int dtype, int param_dtype,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ 1-D layer
  * Same three calls for wtconv/wtconv1d.py:38-82 (two sub-bands, 1/sqrt(2) butterflies). */
 size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass);
@@ -139,6 +153,12 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
                              int B, int C, int N, int K, int levels,
                              int dtype, int param_dtype,
                              void* workspace, size_t workspace_bytes, void* stream);
+
+int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
+                      const wtconv_param_grads* grads,
+                      int B, int C, int N, int K, int levels,
+                      int dtype, int param_dtype,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

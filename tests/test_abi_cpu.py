@@ -27,7 +27,7 @@ def test_header_symbols_are_exported(lib):
     assert declared == set(_lib.EXPORTS), (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.wtconv_abi_version() == 1
+    assert lib.wtconv_abi_version() == _lib.ABI_VERSION == 2
     assert lib.wtconv_max_kernel_size() == 7
 
 
@@ -38,6 +38,10 @@ def test_workspace_sizes(lib):
     assert lib.wtconv2d_workspace_bytes(128, C, 56, 56, K, L, 1) == fwd
     par = lib.wtconv2d_workspace_bytes(128, C, 56, 56, K, L, 2)
     assert par >= 4 * C * ((1 + 4 * L) * K * K + 1)
+    # the one-call backward pass shares one workspace between its two passes
+    assert lib.wtconv2d_workspace_bytes(128, C, 56, 56, K, L, 3) == max(fwd, par)
+    assert lib.wtconv1d_workspace_bytes(64, 64, 4096, K, 4, 3) == max(
+        lib.wtconv1d_workspace_bytes(64, 64, 4096, K, 4, 1), lib.wtconv1d_workspace_bytes(64, 64, 4096, K, 4, 2))
     assert lib.wtconv1d_workspace_bytes(64, 64, 4096, 5, 4, 0) >= 4 * (64 * 9 * 5 + 64)
     assert lib.wtconv2d_workspace_bytes(0, C, 56, 56, K, L, 0) == 0
     assert lib.wtconv2d_workspace_bytes(1, 1, 20000, 20000, K, L, 0) == 0     # plane beyond 2^28 elements
@@ -90,6 +94,22 @@ def test_null_parameter_pointer_rejected(lib):
     rc = lib.wtconv2d_backward_params(0x1000, 0x2000, ctypes.byref(_params(2)), ctypes.byref(g), 1, 2, 8, 8, 5, 2,
                                       0, 0, 0x3000, 1 << 20, None)
     assert rc == -1 and "gradient pointer" in lib.wtconv_last_error().decode()
+
+
+def test_one_call_backward_validates_like_its_passes(lib):
+    """wtconv2d_backward / wtconv1d_backward reject bad arguments before any launch, with the
+    message of the pass that found them."""
+    from wtconv_amd import _lib
+    g = _lib.ParamGrads()
+    rc = lib.wtconv2d_backward(0x1000, 0x2000, 0x3000, ctypes.byref(_params(2)), ctypes.byref(g), 2, 4, 8, 8, 4, 2,
+                               0, 0, 0x4000, 1 << 20, None)
+    assert rc == -1 and "odd and positive" in lib.wtconv_last_error().decode()
+    rc = lib.wtconv1d_backward(0x1000, 0x2000, 0, ctypes.byref(_params(2)), ctypes.byref(g), 1, 2, 64, 5, 2,
+                               0, 0, 0x4000, 1 << 20, None)
+    assert rc == -1 and "null" in lib.wtconv_last_error().decode()
+    rc = lib.wtconv2d_backward(0x1000, 0x2000, 0x3000, ctypes.byref(_params(2)), ctypes.byref(g), 2, 4, 8, 8, 5, 2,
+                               0, 0, 0x4000, 16, None)
+    assert rc == -3 and "workspace" in lib.wtconv_last_error().decode()
 
 
 def test_check_raises_python_exceptions(lib):

@@ -7,8 +7,8 @@ from . import _build
 
 MAX_LEVELS = 5
 F32, BF16 = 0, 1
-PASS_FORWARD, PASS_BACKWARD_INPUT, PASS_BACKWARD_PARAMS = 0, 1, 2
-ABI_VERSION = 1
+PASS_FORWARD, PASS_BACKWARD_INPUT, PASS_BACKWARD_PARAMS, PASS_BACKWARD = 0, 1, 2, 3
+ABI_VERSION = 2
 
 
 class Params(ctypes.Structure):
@@ -35,6 +35,10 @@ EXPORTS["wtconv_static_scratch_bytes"] = (_z, [])
 EXPORTS["wtconv2d_forward_static"] = (_i, [_p, _p, ctypes.POINTER(Params)] + [_i] * 8 + [_p])
 EXPORTS["wtconv2d_backward_params"] = (
     _i, [_p, _p, ctypes.POINTER(Params), ctypes.POINTER(ParamGrads)] + [_i] * 8 + [_p, _z, _p])
+EXPORTS["wtconv2d_backward"] = (
+    _i, [_p, _p, _p, ctypes.POINTER(Params), ctypes.POINTER(ParamGrads)] + [_i] * 8 + [_p, _z, _p])
+EXPORTS["wtconv1d_backward"] = (
+    _i, [_p, _p, _p, ctypes.POINTER(Params), ctypes.POINTER(ParamGrads)] + [_i] * 7 + [_p, _z, _p])
 for _name in ("wtconv1d_forward", "wtconv1d_backward_input"):
     EXPORTS[_name] = (_i, [_p, _p, ctypes.POINTER(Params)] + [_i] * 7 + [_p, _z, _p])
 EXPORTS["wtconv1d_backward_params"] = (

@@ -586,6 +586,11 @@ const char* wtconv_last_error(void) { return g_err; }
 int wtconv_max_kernel_size(void) { return 7; }
 
 size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, int pass) {
+  if (pass == WTCONV_PASS_BACKWARD) {
+    const size_t a = wtconv2d_workspace_bytes(B, C, H, W, K, levels, WTCONV_PASS_BACKWARD_INPUT);
+    const size_t b = wtconv2d_workspace_bytes(B, C, H, W, K, levels, WTCONV_PASS_BACKWARD_PARAMS);
+    return a > b ? a : b;
+  }
   if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
   if (static_cast<long long>(H) * W > kMaxPlaneElems) return 0;
   size_t floats;
@@ -702,7 +707,23 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   return check_launch("wgrad_finish_kernel");
 }
 
+int wtconv2d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
+                      const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels, int dtype,
+                      int param_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  // the two passes run one after the other on the stream and may share the workspace
+  if (int e = wtconv2d_backward_input(grad_out, grad_x, params, B, C, H, W, K, levels, dtype, param_dtype, workspace,
+                                      workspace_bytes, stream))
+    return e;
+  return wtconv2d_backward_params(x, grad_out, params, grads, B, C, H, W, K, levels, dtype, param_dtype, workspace,
+                                  workspace_bytes, stream);
+}
+
 size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass) {
+  if (pass == WTCONV_PASS_BACKWARD) {
+    const size_t a = wtconv1d_workspace_bytes(B, C, N, K, levels, WTCONV_PASS_BACKWARD_INPUT);
+    const size_t b = wtconv1d_workspace_bytes(B, C, N, K, levels, WTCONV_PASS_BACKWARD_PARAMS);
+    return a > b ? a : b;
+  }
   if (B <= 0 || C <= 0 || N <= 0 || K <= 0 || levels <= 0 || levels > kMaxLevels) return 0;
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
@@ -785,6 +806,16 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(256), static_cast<size_t>(nrec) * sizeof(float),
             stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 2, L, K);
   return check_launch("wgrad_finish_kernel");
+}
+
+int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
+                      const wtconv_param_grads* grads, int B, int C, int N, int K, int levels, int dtype,
+                      int param_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = wtconv1d_backward_input(grad_out, grad_x, params, B, C, N, K, levels, dtype, param_dtype, workspace,
+                                      workspace_bytes, stream))
+    return e;
+  return wtconv1d_backward_params(x, grad_out, params, grads, B, C, N, K, levels, dtype, param_dtype, workspace,
+                                  workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -49,6 +49,32 @@ def _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss):
     return pd, conv(base_w), conv(base_b), conv(base_s), [conv(w) for w in wt_ws], [conv(s) for s in wt_ss]
 
 
+_TABLES = {}
+
+
+def _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss):
+    """(param dtype, Params table, tensors kept alive).  Fast path: parameters that already sit
+    on x's device, contiguous, in one kernel dtype are passed as they are, and the table of
+    their addresses is cached under those addresses (a table is nothing but its key)."""
+    pd = base_w.dtype
+    dev = x.device
+    tensors = (base_w, base_s, *wt_ws, *wt_ss) if base_b is None else (base_w, base_s, base_b, *wt_ws, *wt_ss)
+    if pd in _DT:
+        for t in tensors:
+            if t.dtype != pd or t.device != dev or not t.is_contiguous():
+                break
+        else:
+            key = (pd, base_b is not None, *[t.data_ptr() for t in tensors])
+            tab = _TABLES.get(key)
+            if tab is None:
+                if len(_TABLES) > 4096:
+                    _TABLES.clear()
+                tab = _TABLES[key] = _table(_lib.Params, base_w, base_b, base_s, wt_ws, wt_ss)
+            return pd, tab, tensors
+    pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    return pd, _table(_lib.Params, bw, bb, bs, ws, ss), (bw, bb, bs, ws, ss)
+
+
 def _table(cls, base_w, base_b, base_s, wt_ws, wt_ss):
     tab = cls()
     tab.base_weight, tab.base_bias, tab.base_scale = _ptr(base_w), _ptr(base_b), _ptr(base_s)
@@ -111,11 +137,10 @@ def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
         # fp32 kernels run on the exact fp16 values and the result is rounded to fp16 once.
         out, _ = _forward_impl(x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L)
         return out.to(torch.float16), x
-    pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    pd, tab, _keep = _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
     shape = tuple(x.shape)
     with _on_device(x.device):
         out = torch.empty_like(x)
-        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         wsz = _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_FORWARD)
         wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
@@ -140,41 +165,49 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
         g = g.to(x.dtype)
     if not g.is_contiguous():
         g = g.contiguous()
-    pd, bw, bb, bs, ws, ss = _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    pd, tab, _keep = _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    has_bias = base_b is not None
     shape = tuple(x.shape)
     grad_x = None
     grads = [None] * (3 + 2 * L)
     with _on_device(x.device):
-        tab = _table(_lib.Params, bw, bb, bs, ws, ss)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        # one workspace for both passes: they run back to back on one stream
-        wsz = max(_workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_INPUT) if need_x else 0,
-                  _workspace_bytes(lib, dims, shape, K, L, _lib.PASS_BACKWARD_PARAMS) if need_params else 0,
-                  256)
+        which = (_lib.PASS_BACKWARD if need_x and need_params else
+                 _lib.PASS_BACKWARD_INPUT if need_x else _lib.PASS_BACKWARD_PARAMS)
+        wsz = _workspace_bytes(lib, dims, shape, K, L, which)
         wsp = torch.empty(wsz, dtype=torch.uint8, device=x.device)
         dt, pdt = _DT[x.dtype], _DT[pd]
         if need_x:
             grad_x = torch.empty_like(x)
+        if need_params:
+            # one flat fp32 buffer for every gradient: a single allocation and, for bf16
+            # parameters, a single cast afterwards
+            plist = [base_w, base_s] + ([base_b] if has_bias else []) + list(wt_ws) + list(wt_ss)
+            sizes = [t.numel() for t in plist]
+            flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
+            views = flat.split(sizes)
+            nb = 3 if has_bias else 2
+            gtab = _table(_lib.ParamGrads, views[0], views[2] if has_bias else None, views[1],
+                          views[nb:nb + L], views[nb + L:])
+        if need_x and need_params:        # the whole backward pass in one library call
+            fn = lib.wtconv2d_backward if dims == 2 else lib.wtconv1d_backward
+            rc = fn(x.data_ptr(), g.data_ptr(), grad_x.data_ptr(), ctypes.byref(tab), ctypes.byref(gtab), *shape, K, L,
+                    dt, pdt, wsp.data_ptr(), wsz, stream)
+            if rc:
+                _lib.check(rc, "wtconv backward")
+        elif need_x:
             fn = lib.wtconv2d_backward_input if dims == 2 else lib.wtconv1d_backward_input
             rc = fn(g.data_ptr(), grad_x.data_ptr(), ctypes.byref(tab), *shape, K, L, dt, pdt,
                     wsp.data_ptr(), wsz, stream)
             if rc:
                 _lib.check(rc, "wtconv backward_input")
-        if need_params:
-            # one flat fp32 buffer for every gradient: a single allocation and, for bf16
-            # parameters, a single cast afterwards
-            plist = [bw, bs] + ([bb] if bb is not None else []) + list(ws) + list(ss)
-            sizes = [t.numel() for t in plist]
-            flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
-            views = flat.split(sizes)
-            nb = 3 if bb is not None else 2
-            gtab = _table(_lib.ParamGrads, views[0], views[2] if bb is not None else None, views[1],
-                          views[nb:nb + L], views[nb + L:])
+        elif need_params:
             fn = lib.wtconv2d_backward_params if dims == 2 else lib.wtconv1d_backward_params
             rc = fn(x.data_ptr(), g.data_ptr(), ctypes.byref(tab), ctypes.byref(gtab), *shape, K, L, dt, pdt,
                     wsp.data_ptr(), wsz, stream)
             if rc:
                 _lib.check(rc, "wtconv backward_params")
+        if need_params:
             tensors = [base_w, base_s] + ([base_b] if base_b is not None else []) + list(wt_ws) + list(wt_ss)
             out_dt = base_w.dtype
             if all(t.dtype == out_dt for t in tensors):
