@@ -155,6 +155,7 @@ def test_config4_1d_small_batch(hip_device):
     ((1, 2, 8192), 3, 2, True, 1),     # row-resident at the 512-lane limit
     ((1, 2, 20000), 5, 4, True, 1),    # beyond it: tiled kernels, 20 tiles
     ((5, 4, 4096), 5, 4, True, 1),     # several rows per chunk in the parameter-gradient kernel
+    ((35000, 2, 8), 3, 2, True, 1),    # 70 000 short rows: the tiled kernels beyond one 65 535-row grid slice
 ])
 def test_edge_shapes_1d(hip_device, shape, K, L, bias, stride):
     _run_fp32("1d", shape[1], K, L, shape, hip_device, bias=bias, stride=stride, seed=5)
@@ -321,6 +322,93 @@ def test_torch_compile_custom_op(hip_device):
         for n, p in mod.named_parameters():
             if n in eager:
                 assert torch.equal(p.grad, eager[n]), n
+
+
+def test_torch_compile_against_oracle(hip_device):
+    """The compiled layer (opaque operator, registered backward) against the CPU oracle itself,
+    not against the eager HIP run: forward, input gradient and every parameter gradient."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 6, 5, 3, (2, 6, 28, 20))
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 3).to(hip_device)
+    cmod = torch.compile(mod, backend="aot_eager", fullgraph=True)
+    xc = x.to(hip_device).requires_grad_(True)
+    oc = cmod(xc)
+    oc.backward(g.to(hip_device))
+    torch.cuda.synchronize()
+    grads = {n: p.grad.detach().cpu() for n, p in mod.named_parameters() if p.grad is not None}
+    U.compare_all((oc.detach().cpu(), xc.grad.cpu(), grads), U.oracle_run(ref, x, g, torch.float64), U.assert_fp32)
+
+
+def test_gradient_checkpointing(hip_device):
+    """torch.utils.checkpoint around the layer (WTConvNeXt stages offer it, wtconvnext.py:209-210 of the
+    reference): the recomputed forward and the backward through it match the oracle."""
+    from torch.utils.checkpoint import checkpoint
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 8, 5, 2, (2, 8, 14, 14))
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 2).to(hip_device)
+    xd = x.to(hip_device).requires_grad_(True)
+    out = checkpoint(mod, xd, use_reentrant=False)
+    out.backward(g.to(hip_device))
+    torch.cuda.synchronize()
+    grads = {n: p.grad.detach().cpu() for n, p in mod.named_parameters() if p.grad is not None}
+    U.compare_all((out.detach().cpu(), xd.grad.cpu(), grads), U.oracle_run(ref, x, g, torch.float64), U.assert_fp32)
+
+
+def test_converted_checkpoint_runs_on_the_fast_twin(hip_device):
+    """A reference-layout state dict converted with wtconv_amd.convert.reference_to_fast loads into
+    fast_wtconv.wtconv_cuda.WTConv2d (strict) and the HIP layer then matches the oracle that holds
+    the original parameters; converting back recreates the frozen filter banks."""
+    from fast_wtconv.wtconv_cuda import WTConv2d as Fast
+    from wtconv_amd import convert
+    ref, x, g = U.seeded_case("2d", 6, 5, 2, (2, 6, 18, 22))
+    U.randomize_scales(ref)
+    fast = Fast(6, 6, 5, 1, 2, True)
+    missing, unexpected = fast.load_state_dict(convert.reference_to_fast(ref.state_dict()), strict=True)
+    assert not missing and not unexpected
+    fast = fast.to(hip_device)
+    xd = x.to(hip_device).requires_grad_(True)
+    out = fast(xd)
+    out.backward(g.to(hip_device))
+    torch.cuda.synchronize()
+    wo, wdx, wg = U.oracle_run(ref, x, g, torch.float64)
+    U.assert_fp32(out.detach().cpu(), wo, "out")
+    U.assert_fp32(xd.grad.cpu(), wdx, "grad_x")
+    back = convert.fast_to_reference({k: v.detach().cpu() for k, v in fast.state_dict().items()})
+    assert set(back) == set(ref.state_dict())
+    names = {"base_weight": "base_conv.weight", "base_bias": "base_conv.bias", "base_scale": "base_scale.weight",
+             "wt_weights.0": "wavelet_convs.0.weight", "wt_weights.1": "wavelet_convs.1.weight",
+             "wt_scales.0": "wavelet_scale.0.weight", "wt_scales.1": "wavelet_scale.1.weight"}
+    for n, p in fast.named_parameters():
+        U.assert_fp32(p.grad.detach().cpu().reshape(wg[names[n]].shape), wg[names[n]], n)
+
+
+def test_fp32_on_the_matrix_cores_keeps_the_fp32_bar():
+    """WTCONV_MFMA=2 sends fp32 tensors through the MFMA kernels as three bf16 split planes (six
+    products per filter tap): results must hold the fp32 bar.  The switch is read once per process,
+    hence the child process."""
+    import os
+    import subprocess
+    import sys
+    import textwrap
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = textwrap.dedent("""
+        import sys, torch
+        sys.path.insert(0, %r); sys.path.insert(0, %r)
+        import parity_util as U
+        import wtconv
+        dev = torch.device("cuda:0")
+        for C, H, W, L, B in ((8, 56, 56, 3, 3), (6, 28, 28, 3, 5), (5, 14, 14, 2, 7), (4, 7, 7, 2, 9), (3, 33, 17, 4, 2)):
+            ref, x, g = U.seeded_case("2d", C, 5, L, (B, C, H, W))
+            U.randomize_scales(ref)
+            mod = U.copy_to_hip_module(ref, wtconv.WTConv2d, "2d", 5, L)
+            U.compare_all(U.hip_run(mod, x, g, dev), U.oracle_run(ref, x, g, torch.float64), U.assert_fp32)
+        print("ok")
+    """ % (root, os.path.join(root, "tests")))
+    env = dict(os.environ, WTCONV_MFMA="2")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, env=env)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout[-2000:] + r.stderr[-4000:]
 
 
 def test_hip_graph_replay_matches_eager(hip_device):

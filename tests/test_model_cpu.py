@@ -40,3 +40,37 @@ def test_structure_and_init():
     assert set(r.state_dict()) == keys
     out = r(torch.randn(1, 3, 64, 64))
     assert out.shape == (1, 10)
+
+
+def test_drop_path_schedule_and_head_options():
+    """drop_path_rate spreads linearly over all blocks (reference wtconvnext.py:309), is the identity
+    in eval mode and keeps the expectation in training; head_init_scale scales the classifier
+    (wtconvnext.py:483-493); reset_classifier / forward_head(pre_logits) follow the reference's API."""
+    import wtconvnext
+    from oracle import wtconv_ref as R
+    torch.manual_seed(0)
+    m = wtconvnext.wtconvnext_tiny(depths=(1, 2, 1, 1), num_classes=7, drop_path_rate=0.4, head_init_scale=0.5,
+                                   wtconv_class=R.RefWTConv2d)
+    rates = [getattr(b.drop_path, "drop_prob", 0.0) for s in m.stages for b in s.blocks]
+    assert rates == pytest.approx([0.0, 0.1, 0.2, 0.3, 0.4])
+    torch.manual_seed(0)
+    ref = wtconvnext.wtconvnext_tiny(depths=(1, 2, 1, 1), num_classes=7, wtconv_class=R.RefWTConv2d)
+    assert torch.allclose(m.head.fc.weight, 0.5 * ref.head.fc.weight)
+    x = torch.randn(2, 3, 64, 64)
+    m.eval()
+    ref.eval()
+    with torch.no_grad():
+        ref.head.fc.load_state_dict(m.head.fc.state_dict())
+        assert torch.equal(m(x), ref(x))                     # stochastic depth is off in eval mode
+        feats = m.forward_features(x)
+        assert m.forward_head(feats, pre_logits=True).shape == (2, 768)
+    dp = wtconvnext.wtconvnext.DropPath(0.25).train()
+    y = dp(torch.ones(4000, 3))
+    kept = (y[:, 0] != 0).float().mean().item()
+    assert abs(kept - 0.75) < 0.03 and torch.all((y == 0) | (y == 1 / 0.75))
+    m.reset_classifier(3)
+    assert m(x).shape == (2, 3) and m.num_classes == 3
+    m.set_grad_checkpointing(True)
+    m.train()
+    m(x.requires_grad_(True)).sum().backward()
+    assert x.grad is not None

@@ -293,3 +293,85 @@ def test_seeded_default_init_draw_order():
     keys = set(m.state_dict().keys())
     assert {"base_conv.weight", "base_conv.bias", "base_scale.weight", "wavelet_convs.0.weight",
             "wavelet_scale.1.weight", "wt_filter", "iwt_filter"} <= keys
+
+
+def _block_mean_zero_padded(t):
+    """B(t)[i, j] = (sum of the 2 x 2 block of t zero-padded to even sizes) / 4, written out with
+    loops (no conv, no padding helper): the hand-made side of the odd-size check below."""
+    H, W = t.shape
+    h, w = (H + 1) // 2, (W + 1) // 2
+    out = torch.zeros(h, w, dtype=t.dtype)
+    for i in range(h):
+        for j in range(w):
+            s = 0.0
+            for a in (0, 1):
+                for b in (0, 1):
+                    y, x = 2 * i + a, 2 * j + b
+                    if y < H and x < W:          # positions beyond the plane are the zero padding
+                        s = s + t[y, x]
+            out[i, j] = s / 4
+    return out
+
+
+def _upsample_crop(t, H, W):
+    """U(t): every value repeated over its 2 x 2 block, cropped to H x W (loops)."""
+    out = torch.zeros(H, W, dtype=t.dtype)
+    for y in range(H):
+        for x in range(W):
+            out[y, x] = t[y // 2, x // 2]
+    return out
+
+
+@pytest.mark.parametrize("H,W,L", [(5, 7, 2), (6, 10, 3), (7, 7, 3), (9, 4, 2)])
+def test_delta_kernels_odd_sizes_closed_form(H, W, L):
+    """Odd sizes pin the pad side (right/bottom), the per-level padding and the crop of the whole
+    layer: with centre-tap wavelet kernels, unit scales and no base conv the layer is
+        out = x + U(B x) + U U(B B x) + ...   (L - 1 terms)
+    where B is the mean over 2 x 2 blocks of the zero-padded plane and U repeats and crops
+    (reference wtconv2d.py:49-51,66-76).  (6, 10, 3) has an odd level-2 grid (3 x 5), (7, 7, 3) is odd
+    at levels 1 and 3, (9, 4, 2) mixes an odd and an even side."""
+    C, K = 2, 3
+    ref = R.RefWTConv2d(C, C, K, wt_levels=L, bias=True).double()
+    with torch.no_grad():
+        ref.base_conv.weight.zero_()
+        ref.base_conv.bias.zero_()
+        for conv, sc in zip(ref.wavelet_convs, ref.wavelet_scale):
+            conv.weight.zero_()
+            conv.weight[:, 0, K // 2, K // 2] = 1.0
+            sc.weight.fill_(1.0)
+    x = torch.randn(1, C, H, W, dtype=torch.float64)
+    got = ref(x)
+    for c in range(C):
+        want = x[0, c].clone()
+        level = x[0, c]
+        shapes = []
+        for _ in range(L - 1):
+            shapes.append(level.shape)
+            level = _block_mean_zero_padded(level)
+            term = level
+            for (h, w) in reversed(shapes):
+                term = _upsample_crop(term, h, w)
+            want = want + term
+        torch.testing.assert_close(got[0, c], want, rtol=1e-12, atol=1e-12)
+
+
+def test_seeded_default_init_draw_order_1d():
+    """The 1-D layer draws like its 2-D twin: base Conv1d (weight, then bias), then the level convs
+    in order (wtconv1d.py:23-31), against a plain nn.Conv1d sequence under the same seed."""
+    C, K, L = 3, 5, 3
+    torch.manual_seed(0)
+    m = R.RefWTConv1d(C, C, K, wt_levels=L)
+    torch.manual_seed(0)
+    base = torch.nn.Conv1d(C, C, K, padding='same', groups=C, bias=True)
+    lv = [torch.nn.Conv1d(2 * C, 2 * C, K, padding='same', groups=2 * C, bias=False) for _ in range(L)]
+    assert torch.equal(m.base_conv.weight, base.weight) and torch.equal(m.base_conv.bias, base.bias)
+    for i in range(L):
+        assert torch.equal(m.wavelet_convs[i].weight, lv[i].weight)
+        assert torch.all(m.wavelet_scale[i].weight == 0.1)
+    assert torch.all(m.base_scale.weight == 1.0)
+    from wtconv.wtconv1d import WTConv1d
+    torch.manual_seed(0)
+    p = WTConv1d(C, C, K, wt_levels=L)            # the product module draws the same numbers
+    assert torch.equal(p.base_conv.weight, base.weight) and torch.equal(p.base_conv.bias, base.bias)
+    for i in range(L):
+        assert torch.equal(p.wavelet_convs[i].weight, lv[i].weight)

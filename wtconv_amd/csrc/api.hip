@@ -353,8 +353,13 @@ static int run_tile1d(const void* x, void* out, const float* fw, const float* fb
   auto kern = wt1d_tile_kernel<T, K, kTJ1D>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
-  WT_LAUNCH(kern, dim3(pl.ntiles, B * pl.C), dim3(kBlock1D), lds, stream, static_cast<const T*>(x),
-            static_cast<T*>(out), fw, fb, pl);
+  const long long nrows = static_cast<long long>(B) * pl.C;
+  if (nrows > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "batch*channels = %lld is too large", nrows);
+  const unsigned gy = nrows < 65535 ? static_cast<unsigned>(nrows) : 65535u;
+  const unsigned gz = static_cast<unsigned>((nrows + gy - 1) / gy);
+  if (gz > 65535u) return fail(WTCONV_E_UNSUPPORTED, "batch*channels = %lld is too large", nrows);
+  WT_LAUNCH(kern, dim3(pl.ntiles, gy, gz), dim3(kBlock1D), lds, stream, static_cast<const T*>(x),
+            static_cast<T*>(out), fw, fb, pl, static_cast<int>(nrows));
   return check_launch("wt1d_tile_kernel");
 }
 
@@ -522,9 +527,6 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
   int nl = 0, block = 0;
   const bool row_resident = row1d_lanes(N, K, L, &nl, &block);
-  if (!row_resident && static_cast<long long>(B) * C > 65535)
-    return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld exceeds the grid limit 65535", fn,
-                static_cast<long long>(B) * C);
   const Plan1D pl = make_plan1d(C, N, K, L, false, esz, x, out, nullptr);
   const size_t need = wtconv1d_workspace_bytes(B, C, N, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
   if (ws == nullptr || ws_bytes < need)

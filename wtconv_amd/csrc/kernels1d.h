@@ -132,11 +132,13 @@ __device__ __forceinline__ void store_run(T* __restrict__ dst, const float (&v)[
 template <typename T, int K, int TJ>
 __global__ __launch_bounds__(kBlock1D) void wt1d_tile_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                         const float* __restrict__ fw,
-                                                        const float* __restrict__ fb, Plan1D pl) {
+                                                        const float* __restrict__ fb, Plan1D pl, int nrows) {
   WT_SHARED_FLOATS(lds);
   constexpr int R = K / 2;
   constexpr int NO = 2 * TJ;
-  const int row = blockIdx.y;
+  // rows run over gridDim.y and, beyond 65535 of them, gridDim.z (the last z-slice may be ragged)
+  const int row = blockIdx.y + blockIdx.z * gridDim.y;
+  if (row >= nrows) return;
   const int c = row % pl.C;
   const int t0 = blockIdx.x * pl.T;
   const int NF = 1 + 2 * pl.L;
