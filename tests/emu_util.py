@@ -13,7 +13,7 @@ EXE = os.path.join(BUILD_DIR, "emu_driver")
 SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(ROOT, "wtconv_amd", "csrc", "mfma2d.hip"),
            os.path.join(EMU_DIR, "emu_driver.cpp")]
 DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
-                  ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h",
+                  ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h", "kernels2d_mfma_wgrad.h",
                    "kernels2d_stream.h", "mfma2d.h", "plan.h")] + [
     os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
 
@@ -26,7 +26,7 @@ def build(force=False):
             return EXE
     # -O0 -g1: the run time is dominated by thread creation, the build time by optimisation
     cmd = ["g++", "-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined",
-           "-fno-sanitize-recover=undefined", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
+           "-fno-sanitize-recover=undefined", "-static-libasan", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
            *SOURCES, "-pthread", "-o", EXE]
     subprocess.run(cmd, check=True, cwd=ROOT)
     return EXE
@@ -61,7 +61,6 @@ def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, 
             f.write(b"".join(parts))
         env = dict(os.environ)
         env["ASAN_OPTIONS"] = "detect_leaks=0"
-        env.pop("LD_PRELOAD", None)
         env.pop("WT_EMU_LDS_LIMIT", None)
         if lds_limit is not None:
             env["WT_EMU_LDS_LIMIT"] = str(int(lds_limit))

@@ -598,6 +598,9 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     int bchunk, nchunk;
+    // the dtype is not an argument here: room for the bf16 matrix-core kernel's partial sums as well
+    const Mfma2dWgradQuery mq = mfma2d_wgrad_query(B, C, H, W, K, levels, WTCONV_BF16);
+    const size_t mfloats = mq.ok ? mq.ws_bytes / sizeof(float) : 0;
     if (wgrad_fits_lds(B, C, H, W, K, levels)) {
       wgrad_chunks(B, C, wgrad_planes_per_iter(B, H, W, K, levels), kWgradResident, &bchunk, &nchunk);
       floats = static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1);
@@ -606,6 +609,7 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
       floats = round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1)) +
                2 * make_stream2d(B, C, H, W, levels).floats;
     }
+    if (mfloats > floats) floats = mfloats;
   } else {
     // the dtype is not an argument here: size for the larger of the two (fp32 tensors take
     // three split tables) whenever either could run on the matrix-core kernels
@@ -680,7 +684,11 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   int bchunk, nchunk;
   float* partial = static_cast<float*>(workspace);
   int e;
-  if (wgrad_fits_lds(B, C, H, W, K, L)) {
+  const Mfma2dWgradQuery mq = mfma2d_wgrad_query(B, C, H, W, K, L, dtype);
+  if (mq.ok) {
+    nchunk = mq.nchunk;
+    e = mfma2d_wgrad_pass(fn, x, grad_out, partial, B, C, H, W, K, L, stream);
+  } else if (wgrad_fits_lds(B, C, H, W, K, L)) {
     const int pb = wgrad_planes_per_iter(B, H, W, K, L);
     Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
     finish_wgrad_plan(&pl, K);

@@ -20,4 +20,16 @@ Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype);
 int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
                 int K, int L, int dtype, int pdtype, hipStream_t stream, int flip);
 
+// Parameter gradients of bf16 tensors: whether the shape runs on the MFMA kernel, and the size of the
+// per-chunk partial sums it leaves in the workspace for wgrad_finish_kernel (`nchunk` records per channel).
+struct Mfma2dWgradQuery {
+  bool ok;
+  int nchunk;
+  size_t ws_bytes;
+};
+Mfma2dWgradQuery mfma2d_wgrad_query(int B, int C, int H, int W, int K, int L, int dtype);
+
+int mfma2d_wgrad_pass(const char* fn, const void* x, const void* grad_out, float* partial, int B, int C, int H, int W,
+                      int K, int L, hipStream_t stream);
+
 }  // namespace wt

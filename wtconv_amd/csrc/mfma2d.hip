@@ -6,6 +6,7 @@
 #include "common.h"
 #include "host_util.h"
 #include "kernels2d_mfma.h"
+#include "kernels2d_mfma_wgrad.h"
 #include "mfma2d.h"
 
 namespace wt {
@@ -197,6 +198,122 @@ int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* p
                    (reinterpret_cast<uintptr_t>(out) & mask) == 0;
   return dtype == WTCONV_F32 ? launch_mfma_nbl<float, 3>(nbl, vec, x, out, a, pl, stream)
                              : launch_mfma_nbl<bf16_t, 1>(nbl, vec, x, out, a, pl, stream);
+}
+
+// ---- parameter gradients ---------------------------------------------------------------------
+namespace {
+
+constexpr int kWgradLdsPair = 80 * 1024;      // two workgroups of four waves per CU below this, else one of eight waves
+
+struct WKey {
+  int B, C, H, W, L;
+  bool operator==(const WKey& o) const { return B == o.B && C == o.C && H == o.H && W == o.W && L == o.L; }
+};
+struct WKeyHash {
+  size_t operator()(const WKey& k) const {
+    size_t h = 1469598103934665603ull;
+    for (int v : {k.B, k.C, k.H, k.W, k.L}) h = (h ^ static_cast<size_t>(v)) * 1099511628211ull;
+    return h;
+  }
+};
+struct WVal { bool ok; WPlan pl; int nw, compact, bchunk, nchunk; };
+
+// Planes per unit: up to one 4x4 block per thread of four waves, within the LDS that leaves room for two
+// workgroups per CU; a single plane beyond that runs as one workgroup of eight waves per CU.
+bool choose_wplan(int B, int C, int H, int W, int L, WVal* v) {
+  const int bpp0 = ceil_div(H, 4) * ceil_div(W, 4);
+  int pb = kMfmaBlock / bpp0;
+  if (pb < 1 || W > 64) return false;
+  if (pb > B) pb = B;
+  if (static_cast<long long>(pb) * C * H * W > 0x7fffffffLL) return false;
+  WPlan pl;
+  bool compact = false;
+  for (;; --pb) {
+    if (!make_wplan_geometry(H, W, L, pb, 512, false, &pl)) return false;
+    if (pl.lds_bytes <= kWgradLdsPair || pb == 1) break;
+  }
+  if (pl.lds_bytes > kWgradLdsPair) {
+    WPlan cp;
+    if (make_wplan_geometry(H, W, L, pb, 512, true, &cp) && cp.lds_bytes <= kWgradLdsPair) { pl = cp; compact = true; }
+  }
+  if (static_cast<size_t>(pl.lds_bytes) > lds_budget()) return false;
+  pl.B = B; pl.C = C;
+  v->pl = pl;
+  v->compact = compact;
+  v->nw = pl.lds_bytes <= kWgradLdsPair ? 4 : 8;
+  wgrad_chunks(B, C, pb, compute_units() * (v->nw == 4 ? 2 : 1), &v->bchunk, &v->nchunk);
+  return true;
+}
+
+// Shape-only part of the plan (pointer alignment is applied per call).
+const WVal& wplan_cached(int B, int C, int H, int W, int L) {
+  static thread_local std::unordered_map<WKey, WVal, WKeyHash> cache;
+  const WKey key = {B, C, H, W, L};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    if (cache.size() > 4096) cache.clear();
+    WVal v = {};
+    v.ok = choose_wplan(B, C, H, W, L, &v);
+    it = cache.emplace(key, v).first;
+  }
+  return it->second;
+}
+
+struct WgradArgs { const void* x; const void* g; float* partial; int K, bchunk, nchunk; };
+
+template <int L, int NW, typename Geo>
+int launch_wgrad(const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
+  auto kern = wt2d_mfma_wgrad_kernel<L, NW, Geo>;
+  const size_t lds = static_cast<size_t>(pl.lds_bytes);
+  if (int e = allow_lds(kern, lds)) return e;
+  WT_LAUNCH(kern, dim3(pl.C, a.nchunk), dim3(NW * 64), lds, stream, static_cast<const bf16_t*>(a.x),
+            static_cast<const bf16_t*>(a.g), a.partial, pl, a.K, a.bchunk);
+  return check_launch("wt2d_mfma_wgrad_kernel");
+}
+
+template <int L>
+int launch_wgrad_l(int nw, bool compact, const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
+#ifndef WT_EMULATE
+  // plane shapes of the WTConvNeXt stages: geometry as a compile-time constant
+#define WT_TRY(H_, L_, PB_, NW_, CMP_) \
+  if (L == L_ && pl.H == H_ && pl.W == H_ && pl.pb == PB_ && nw == NW_ && compact == CMP_) \
+    return launch_wgrad<L_, NW_, WGeoStatic<H_, H_, L_, PB_, 512, CMP_>>(a, pl, stream);
+  WT_TRY(56, 3, 1, 4, true) WT_TRY(28, 3, 3, 4, false) WT_TRY(14, 2, 12, 4, false) WT_TRY(7, 2, 24, 4, false)
+  WT_TRY(56, 5, 1, 8, false) WT_TRY(28, 4, 2, 4, false) WT_TRY(14, 3, 8, 4, false)
+#undef WT_TRY
+#endif
+  return nw == 8 ? launch_wgrad<L, 8, WGeoRuntime>(a, pl, stream) : launch_wgrad<L, 4, WGeoRuntime>(a, pl, stream);
+}
+
+}  // namespace
+
+Mfma2dWgradQuery mfma2d_wgrad_query(int B, int C, int H, int W, int K, int L, int dtype) {
+  Mfma2dWgradQuery r = {false, 0, 0};
+  if (mfma_mode() <= 0 || dtype != WTCONV_BF16 || K > 5 || L < 1 || L > kMaxLevels) return r;
+  if (C > 65535) return r;
+  const WVal& v = wplan_cached(B, C, H, W, L);
+  if (!v.ok || v.nchunk > 65535) return r;
+  r.ok = true;
+  r.nchunk = v.nchunk;
+  r.ws_bytes = static_cast<size_t>(v.nchunk) * C * ((1 + 4 * L) * K * K + 1) * sizeof(float);
+  return r;
+}
+
+int mfma2d_wgrad_pass(const char* fn, const void* x, const void* grad_out, float* partial, int B, int C, int H, int W,
+                      int K, int L, hipStream_t stream) {
+  const WVal& v = wplan_cached(B, C, H, W, L);
+  if (!v.ok) return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
+  WPlan pl = v.pl;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(grad_out)) & 7u) == 0;
+  pl.vec = (W % 4 == 0) && aligned;
+  const WgradArgs a = {x, grad_out, partial, K, v.bchunk, v.nchunk};
+  switch (L) {
+    case 1: return launch_wgrad_l<1>(v.nw, v.compact != 0, a, pl, stream);
+    case 2: return launch_wgrad_l<2>(v.nw, v.compact != 0, a, pl, stream);
+    case 3: return launch_wgrad_l<3>(v.nw, v.compact != 0, a, pl, stream);
+    case 4: return launch_wgrad_l<4>(v.nw, v.compact != 0, a, pl, stream);
+    default: return launch_wgrad_l<5>(v.nw, v.compact != 0, a, pl, stream);
+  }
 }
 
 }  // namespace wt
