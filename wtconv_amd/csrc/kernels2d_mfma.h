@@ -26,15 +26,7 @@ namespace wt {
 
 constexpr int kFragEntries = 21;     // 5 kernel rows x 4 column shifts, then one all-zero entry
 constexpr int kMfmaBlock = 256;
-constexpr int kDivShift = 20;
-#ifndef WT_MF_WHATIF
-#define WT_MF_WHATIF 0
-#endif
-#ifndef WT_MF_TICK
-#define WT_MF_TICK_INIT() do {} while (0)
-#define WT_MF_TICK(k) do {} while (0)
-#define WT_MF_TICK_FLUSH() do {} while (0)
-#endif        // magic reciprocals: exact for dividends < 4096, divisors <= 256
+constexpr int kDivShift = 20;        // magic reciprocals: exact for dividends < 4096, divisors <= 256
 
 struct MPlan {
   int B, C, H, W, L;
@@ -317,6 +309,11 @@ __device__ __forceinline__ void fold_entry(const ParamTable& p, int pdtype, int 
 template <typename T> struct PixRow;
 template <> struct PixRow<float> { float4 v; };
 template <> struct PixRow<bf16_t> { uint2 v; };
+// bf16 pixels fetched one by one (rows that are not whole aligned vectors): each in a register of its own, as
+// it comes from memory -- nothing is computed on them before use, so all the loads of a block stay in flight.
+struct PixRowU { uint32_t e[4]; };
+template <typename T, bool VEC> struct PixSel { using type = PixRow<T>; };
+template <> struct PixSel<bf16_t, false> { using type = PixRowU; };
 
 __device__ __forceinline__ void pix_zero(PixRow<float>& r) { r.v.x = r.v.y = r.v.z = r.v.w = 0.f; }
 __device__ __forceinline__ void pix_zero(PixRow<bf16_t>& r) { r.v.x = r.v.y = 0u; }
@@ -329,6 +326,20 @@ __device__ __forceinline__ void pix_set(PixRow<bf16_t>& r, int i, bf16_t v) {
   const uint32_t u = static_cast<uint32_t>(v) << ((i & 1) * 16);
   if (i < 2) r.v.x |= u; else r.v.y |= u;
 }
+__device__ __forceinline__ void pix_zero(PixRowU& r) { r.e[0] = r.e[1] = r.e[2] = r.e[3] = 0u; }
+__device__ __forceinline__ void pix_load4(PixRowU&, const bf16_t*) {}      // (never taken: vector rows use PixRow)
+__device__ __forceinline__ void pix_set(PixRowU& r, int i, bf16_t v) { r.e[i] = v; }
+__device__ __forceinline__ void pix_get(const PixRowU& r, float (&f)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r.e[i] << 16);
+}
+// the four bf16 of a row as two packed words
+__device__ __forceinline__ uint2 pix_words(const PixRow<bf16_t>& r) { return r.v; }
+__device__ __forceinline__ uint2 pix_words(const PixRowU& r) {
+  uint2 w; w.x = r.e[0] | (r.e[1] << 16); w.y = r.e[2] | (r.e[3] << 16);
+  return w;
+}
+__device__ __forceinline__ uint2 pix_words(const PixRow<float>&) { uint2 w; w.x = w.y = 0u; return w; }   // (never taken)
 __device__ __forceinline__ void pix_get(const PixRow<float>& r, float (&f)[4]) {
   f[0] = r.v.x; f[1] = r.v.y; f[2] = r.v.z; f[3] = r.v.w;
 }
@@ -493,7 +504,7 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   const int u_begin = static_cast<int>(static_cast<long long>(blockIdx.x) * pl.nunits / G);
   const int u_end = static_cast<int>(static_cast<long long>(blockIdx.x + 1) * pl.nunits / G);
 
-  PixRow<T> pf[NBL][4];
+  typename PixSel<T, VEC>::type pf[NBL][4];
   auto fetch = [&](int u) {
     const int c = u / upc;
     const int b0 = (u - c * upc) * pb;
@@ -523,10 +534,8 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   Frag ra0t[NR], ra0b[NR], ra1t[4][NR], ra1b[4][NR];     // resident fragments (RES only)
   int cur_c = -1;
   float bias = 0.f;
-  WT_MF_TICK_INIT();
 #pragma unroll 1
   for (int u = u_begin; u < u_end; ++u) {
-    WT_MF_TICK(0);
     const int c = u / upc;
     const int b0 = (u - c * upc) * pb;
     const int np = B - b0 < pb ? B - b0 : pb;      // planes of this unit that exist
@@ -563,7 +572,6 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
     // ---- commit: pixels -> level-0 planes; analysis levels 1 and 2 from registers
 #pragma unroll
     for (int i = 0; i < NBL; ++i) {
-      if (WT_MF_WHATIF == 3) { if (pf[i][0].v.x == 12345) lds_st<float>(lds, 0, 1.f); continue; }
       if (!(c_mask[i] & 0x100u)) continue;
       float v[4][4];
 #pragma unroll
@@ -572,8 +580,9 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
       for (int r = 0; r < 4; ++r) {
         uint32_t w0[NS], w1[NS];
         if constexpr (NS == 1 && sizeof(T) == 2) {
-          w0[0] = pf[i][r].v.x;      // the values are bf16 already
-          w1[0] = pf[i][r].v.y;
+          const uint2 w = pix_words(pf[i][r]);      // the values are bf16 already
+          w0[0] = w.x;
+          w1[0] = w.y;
         } else {
           split_pair<NS>(v[r][0], v[r][1], w0);
           split_pair<NS>(v[r][2], v[r][3], w1);
@@ -621,10 +630,8 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
         if (L >= 3) lds_st<float>(lds, c_ll[i], cf[0]);
       }
     }
-    WT_MF_TICK(1);
     if (u + 1 < u_end) fetch(u + 1);
     WT_LDS_BARRIER();
-    WT_MF_TICK(2);
 
     // ---- analysis levels 3..L from the raw LL of the level above (fp32 in LDS)
     levels_up<Geo, 3>(L, [&](auto lc) {
@@ -658,11 +665,9 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
       WT_LDS_BARRIER();
     });
 
-    WT_MF_TICK(3);
     // ---- stage 1: the last wave runs levels L..2 (conv + inverse Haar -> Z_l), the others the base
     // conv and, when every wave has at most one level-1 tile, the detail sub-bands of that tile
     const int base_waves = L >= 2 ? 3 : 4;
-    if (WT_MF_WHATIF >= 2) { WT_LDS_BARRIER(); continue; }
     // level-1 convolution of sub-band s of a tile into acc (resident or table fragments)
     auto conv1 = [&](const TileLane& tl, int s, Acc& acc) {
       Frag bt[NS], bb[NS];
@@ -774,14 +779,11 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
         for (int s = 1; s < 4; ++s) conv1(tl1, s, acc1[s]);
       }
     }
-    WT_MF_TICK(4);
     WT_LDS_BARRIER();
-    WT_MF_TICK(5);
 
     // ---- stage 2: level 1 (conv, inverse Haar), plus the base conv from Z_1, to HBM
-    if (WT_MF_WHATIF != 1) {
+    {
       WT_WAIT_VMEM();       // the prefetch has landed; the stores below then drain behind the next unit's work
-      WT_MF_TICK(6);
       T* obase = out + (static_cast<size_t>(b0) * C + c) * HW;
 #pragma unroll 1
       for (int t = wave; t < ntile1; t += 4) {
@@ -847,11 +849,8 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
         }
       }
     }
-    WT_MF_TICK(7);
     WT_LDS_BARRIER();
-    WT_MF_TICK(8);
   }
-  WT_MF_TICK_FLUSH();
 }
 
 }  // namespace wt

@@ -53,10 +53,7 @@ struct WPlan {
   int llxoff[kMaxLevels + 1], llgoff[kMaxLevels + 1], llpl[kMaxLevels + 1];   // fp32 raw LL, 2 <= l < L
   int zero_off;
   int lds_bytes;
-  int vec;                           // plane rows are whole aligned 4-element vectors
 };
-
-constexpr int kWgRedFloats = 25 * (1 + kMaxLevels) + 1;    // taps of the base conv and of one sub-band per level, sum of grad_out
 
 // Shape-dependent part of the plan (constexpr: compile-time constant for the common shapes).
 // `compact` gives the narrow levels from 2 on rows of an even number of 16-byte units (two-way bank conflicts
@@ -111,7 +108,8 @@ constexpr bool make_wplan_geometry(int H, int W, int L, int pb, int nthreads, bo
   }
   pl.zero_off = off;   // 64 bytes that stay zero: a dY window may end a few elements past its image, idle lane groups read A here
   off += 64;
-  if (off < 8 * kWgRedFloats * 4) off = 8 * kWgRedFloats * 4;     // the final reduction reuses the images
+  // the final reduction reuses the images: per wave the five diagonals of 12 elements of 5 (1 + L) tiles
+  if (off < 8 * ((1 + L) * 5 * 5 * kWgRowStep * 4 + 4)) off = 8 * ((1 + L) * 5 * 5 * kWgRowStep * 4 + 4);
   pl.lds_bytes = rup(off, 16);
   *out = pl;
   return true;
@@ -179,15 +177,15 @@ __device__ __forceinline__ void corr_mma(const CorrTile<NX>& t, Acc (&d)[5]) {
 
 // Grid (C, nchunk): workgroup (c, k) sums over batch items [k * bchunk, (k + 1) * bchunk) of channel c.
 // NW = 4 or 8 waves per workgroup.
-template <int L, int NW, typename Geo>
-__global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 2)
+template <int L, int NW, bool VEC, typename Geo>
+__global__ void __launch_bounds__(NW * 64, 2)
 wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ g, float* __restrict__ partial,
                        const WPlan plarg, int K, int bchunk) {
   const WPlan pl = [&]() {
     if constexpr (Geo::kStatic) {
       constexpr WPlan gp = Geo::plan();
       WPlan p = gp;
-      p.B = plarg.B; p.C = plarg.C; p.vec = plarg.vec;
+      p.B = plarg.B; p.C = plarg.C;
       return p;
     } else {
       return plarg;
@@ -203,12 +201,6 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
   const int c = blockIdx.x;
   const int b_begin = blockIdx.y * bchunk;
   const int b_end = b_begin + bchunk < B ? b_begin + bchunk : B;
-
-  for (int o = tid * 16; o < pl.lds_bytes; o += NT * 16) {
-    uint4 z; z.x = z.y = z.z = z.w = 0u;
-    lds_st<uint4>(lds, o, z);
-  }
-  WT_LDS_BARRIER();
 
   // ---- commit role: one 4x4 pixel block per thread of four waves -- of x and of grad_out, or with eight
   // waves of x in the first four and of grad_out in the others
@@ -239,7 +231,8 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
   const int xsub2 = pl.xsub[L >= 2 ? 2 : 0], gsub2 = pl.gsub[L >= 2 ? 2 : 0];
   const int llx2 = pl.llxoff[L >= 3 ? 2 : 0], llg2 = pl.llgoff[L >= 3 ? 2 : 0];
 
-  PixRow<bf16_t> px[4], pg[kSplitCommit ? 1 : 4];
+  using Pix = typename PixSel<bf16_t, VEC>::type;
+  Pix px[4], pg[kSplitCommit ? 1 : 4];
   const bf16_t* src0 = (kSplitCommit && half) ? g : x;
   auto fetch = [&](int b0) {
     const size_t base = (static_cast<size_t>(b0) * C + c) * HW;
@@ -251,7 +244,7 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
       if (plane_ok && (cmask >> r & 1u)) {
         const bf16_t* sx = src0 + base + c_goff + r * W;
         const bf16_t* sg = g + base + c_goff + r * W;
-        if (pl.vec) {
+        if constexpr (VEC) {
           if (cmask & 16u) {
             pix_load4(px[r], sx);
             if constexpr (!kSplitCommit) pix_load4(pg[r], sg);
@@ -269,8 +262,15 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
   };
   if (b_begin < b_end) fetch(b_begin);
 
+  // halos, padding rows and the rows of planes past the batch stay zero from here on
+  for (int o = tid * 16; o < pl.lds_bytes; o += NT * 16) {
+    uint4 z; z.x = z.y = z.z = z.w = 0u;
+    lds_st<uint4>(lds, o, z);
+  }
+  WT_LDS_BARRIER();
+
   // pixels -> level-0 image; levels 1 and 2 from registers (N1 split planes each); the raw LL of level 2 to `llo`
-  auto commit = [&](const PixRow<bf16_t> (&pr)[4], int o0, int pitch0, bool pair64, int o1, int pitch1, int sub1, int o2,
+  auto commit = [&](const Pix (&pr)[4], int o0, int pitch0, bool pair64, int o1, int pitch1, int sub1, int o2,
                     int sub2, int llo, float& llsum, auto n1) {
     constexpr int N1 = decltype(n1)::value;
     float v[4][4];
@@ -278,11 +278,12 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     for (int r = 0; r < 4; ++r) pix_get(pr[r], v[r]);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
+      const uint2 w = pix_words(pr[r]);
       if (pair64) {
-        lds_st<uint2>(lds, o0 + r * pitch0 * 2, pr[r].v);
+        lds_st<uint2>(lds, o0 + r * pitch0 * 2, w);
       } else {
-        lds_st<uint32_t>(lds, o0 + r * pitch0 * 2, pr[r].v.x);
-        lds_st<uint32_t>(lds, o0 + r * pitch0 * 2 + 4, pr[r].v.y);
+        lds_st<uint32_t>(lds, o0 + r * pitch0 * 2, w.x);
+        lds_st<uint32_t>(lds, o0 + r * pitch0 * 2 + 4, w.y);
       }
     }
     float ll1[2][2];
@@ -459,57 +460,54 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     WT_LDS_BARRIER();
   }
 
-  // ---- extract the taps: tap (kh, kw) = sum over n < 12 of D_kw[n + kh][n]; lane (n, q) holds D[4q + r][n]
+  // ---- taps: tap (kh, kw) of a filter = sum over n < 12 of D_kw[n + kh][n]; lane (n, q) holds D[4q + r][n].
+  // Every wave leaves the five diagonals of its tiles in LDS (the images are dead after the last barrier),
+  // then the threads sum them: over n, and over the waves that shared a filter.
   const int KK = K * K;
   const int nrec = (1 + 4 * L) * KK + 1;
   float* rec = partial + (static_cast<size_t>(blockIdx.y) * C + c) * nrec;
-  float* red = reinterpret_cast<float*>(lds) + wave * kWgRedFloats;        // the images are dead after the last barrier
-  auto diag = [&](const Acc& d, int kh) {
-    float v = 0.f;
+  constexpr int kBand = 5 * kWgRowStep * 4;                 // bytes of the diagonals of one tile
+  constexpr int kWaveBand = (1 + L) * 5 * kBand;            // ... of one wave: tiles [filter][kw]
+  auto put = [&](const Acc& d, int slot) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (4 * q + r - n == kh && n < kWgRowStep) v += d.v[r];
-    return wave_sum(v);
-  };
-#pragma unroll 1
-  for (int kh = 0; kh < 5; ++kh)
-#pragma unroll
-    for (int kw = 0; kw < 5; ++kw) {
-      const float vb = diag(db[kw], kh);
-      if (lane == 0) red[kh * 5 + kw] = vb;
-#pragma unroll
-      for (int l = 1; l <= L; ++l) {
-        const float v = diag(dl[l - 1][kw], kh);
-        if (lane == 0) red[25 * l + kh * 5 + kw] = v;
-      }
+    for (int r = 0; r < 4; ++r) {
+      const int kh = 4 * q + r - n;
+      if (kh >= 0 && kh < 5 && n < kWgRowStep) lds_st<float>(lds, wave * kWaveBand + slot * kBand + (kh * kWgRowStep + n) * 4, d.v[r]);
     }
+  };
+#pragma unroll
+  for (int kw = 0; kw < 5; ++kw) {
+    put(db[kw], kw);
+#pragma unroll
+    for (int l = 1; l <= L; ++l) put(dl[l - 1][kw], l * 5 + kw);
+  }
   const float gs = wave_sum(gsum);
-  if (lane == 0) red[25 * (1 + L)] = gs;
+  if (lane == 0) lds_st<float>(lds, NW * kWaveBand + wave * 4, gs);
   WT_LDS_BARRIER();
-  const float* all = reinterpret_cast<const float*>(lds);
-  // base conv and sum of grad_out: over all waves; level l, sub-band s: over the waves s, s + 4, ...
   for (int i = tid; i < 25 * (1 + 4 * L) + 1; i += NT) {
     float v = 0.f;
-    if (i < 25 || i == 25 * (1 + 4 * L)) {
-      const int slot = i < 25 ? i : 25 * (1 + L);
+    if (i == 25 * (1 + 4 * L)) {
 #pragma unroll
-      for (int wv = 0; wv < NW; ++wv) v += all[wv * kWgRedFloats + slot];
-      if (i < 25) {
-        const int t = tap_of_frame(i / 5, i % 5, K);
-        if (t >= 0) rec[t] = v;
-      } else {
-        rec[nrec - 1] = v;
-      }
-    } else {
-      const int f = (i - 25) / 25, tap = (i - 25) - 25 * f;        // f = 4 (l - 1) + s
-      const int l = (f >> 2) + 1, s = f & 3;
-#pragma unroll
-      for (int hf = 0; hf < NH; ++hf) v += all[(s + 4 * hf) * kWgRedFloats + 25 * l + tap];
-      float sc = 1.f;
-      for (int k = 0; k < l; ++k) sc *= 0.25f;      // both pyramids were left unnormalised: 2^l each
-      const int t = tap_of_frame(tap / 5, tap % 5, K);
-      if (t >= 0) rec[(1 + f) * KK + t] = v * sc;
+      for (int wv = 0; wv < NW; ++wv) v += lds_ld<float>(lds, NW * kWaveBand + wv * 4);
+      rec[nrec - 1] = v;
+      continue;
     }
+    const int f = i / 25, tap = i - 25 * f;          // f = 0: base conv; else 1 + 4 (l - 1) + s
+    const int kh = tap / 5, kw = tap - 5 * kh;
+    const int l = f == 0 ? 0 : ((f - 1) >> 2) + 1;
+    const int w0 = f == 0 ? 0 : ((f - 1) & 3), wstep = f == 0 ? 1 : 4;      // base conv: every wave; sub-band s: waves s, s + 4, ...
+    const int o = (l * 5 + kw) * kBand + kh * kWgRowStep * 4;
+    for (int wv = w0; wv < NW; wv += wstep) {
+      float4 t[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) t[j] = lds_ld<float4>(lds, wv * kWaveBand + o + 16 * j);
+      v += ((t[0].x + t[0].y) + (t[0].z + t[0].w)) + ((t[1].x + t[1].y) + (t[1].z + t[1].w)) +
+           ((t[2].x + t[2].y) + (t[2].z + t[2].w));
+    }
+    float sc = 1.f;
+    for (int k = 0; k < l; ++k) sc *= 0.25f;        // both pyramids were left unnormalised: 2^l each
+    const int t = tap_of_frame(kh, kw, K);
+    if (t >= 0) rec[f * KK + t] = v * sc;
   }
 }
 

@@ -261,9 +261,9 @@ const WVal& wplan_cached(int B, int C, int H, int W, int L) {
 
 struct WgradArgs { const void* x; const void* g; float* partial; int K, bchunk, nchunk; };
 
-template <int L, int NW, typename Geo>
+template <int L, int NW, bool VEC, typename Geo>
 int launch_wgrad(const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
-  auto kern = wt2d_mfma_wgrad_kernel<L, NW, Geo>;
+  auto kern = wt2d_mfma_wgrad_kernel<L, NW, VEC, Geo>;
   const size_t lds = static_cast<size_t>(pl.lds_bytes);
   if (int e = allow_lds(kern, lds)) return e;
   WT_LAUNCH(kern, dim3(pl.C, a.nchunk), dim3(NW * 64), lds, stream, static_cast<const bf16_t*>(a.x),
@@ -272,17 +272,19 @@ int launch_wgrad(const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
 }
 
 template <int L>
-int launch_wgrad_l(int nw, bool compact, const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
+int launch_wgrad_l(int nw, bool compact, bool vec, const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
 #ifndef WT_EMULATE
   // plane shapes of the WTConvNeXt stages: geometry as a compile-time constant
 #define WT_TRY(H_, L_, PB_, NW_, CMP_) \
-  if (L == L_ && pl.H == H_ && pl.W == H_ && pl.pb == PB_ && nw == NW_ && compact == CMP_) \
-    return launch_wgrad<L_, NW_, WGeoStatic<H_, H_, L_, PB_, 512, CMP_>>(a, pl, stream);
+  if (L == L_ && pl.H == H_ && pl.W == H_ && pl.pb == PB_ && nw == NW_ && compact == CMP_ && vec == (H_ % 4 == 0)) \
+    return launch_wgrad<L_, NW_, H_ % 4 == 0, WGeoStatic<H_, H_, L_, PB_, 512, CMP_>>(a, pl, stream);
   WT_TRY(56, 3, 1, 4, true) WT_TRY(28, 3, 3, 4, false) WT_TRY(14, 2, 12, 4, false) WT_TRY(7, 2, 24, 4, false)
   WT_TRY(56, 5, 1, 8, false) WT_TRY(28, 4, 2, 4, false) WT_TRY(14, 3, 8, 4, false)
 #undef WT_TRY
 #endif
-  return nw == 8 ? launch_wgrad<L, 8, WGeoRuntime>(a, pl, stream) : launch_wgrad<L, 4, WGeoRuntime>(a, pl, stream);
+  if (vec)
+    return nw == 8 ? launch_wgrad<L, 8, true, WGeoRuntime>(a, pl, stream) : launch_wgrad<L, 4, true, WGeoRuntime>(a, pl, stream);
+  return nw == 8 ? launch_wgrad<L, 8, false, WGeoRuntime>(a, pl, stream) : launch_wgrad<L, 4, false, WGeoRuntime>(a, pl, stream);
 }
 
 }  // namespace
@@ -305,14 +307,14 @@ int mfma2d_wgrad_pass(const char* fn, const void* x, const void* grad_out, float
   if (!v.ok) return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
   WPlan pl = v.pl;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(grad_out)) & 7u) == 0;
-  pl.vec = (W % 4 == 0) && aligned;
+  const bool vec = (W % 4 == 0) && aligned;
   const WgradArgs a = {x, grad_out, partial, K, v.bchunk, v.nchunk};
   switch (L) {
-    case 1: return launch_wgrad_l<1>(v.nw, v.compact != 0, a, pl, stream);
-    case 2: return launch_wgrad_l<2>(v.nw, v.compact != 0, a, pl, stream);
-    case 3: return launch_wgrad_l<3>(v.nw, v.compact != 0, a, pl, stream);
-    case 4: return launch_wgrad_l<4>(v.nw, v.compact != 0, a, pl, stream);
-    default: return launch_wgrad_l<5>(v.nw, v.compact != 0, a, pl, stream);
+    case 1: return launch_wgrad_l<1>(v.nw, v.compact != 0, vec, a, pl, stream);
+    case 2: return launch_wgrad_l<2>(v.nw, v.compact != 0, vec, a, pl, stream);
+    case 3: return launch_wgrad_l<3>(v.nw, v.compact != 0, vec, a, pl, stream);
+    case 4: return launch_wgrad_l<4>(v.nw, v.compact != 0, vec, a, pl, stream);
+    default: return launch_wgrad_l<5>(v.nw, v.compact != 0, vec, a, pl, stream);
   }
 }
 
