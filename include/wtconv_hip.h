@@ -26,7 +26,7 @@ extern "C" {
 #endif
 
 #define WTCONV_MAX_LEVELS 5
-#define WTCONV_ABI_VERSION 2
+#define WTCONV_ABI_VERSION 3
 
 enum { WTCONV_F32 = 0, WTCONV_BF16 = 1 };
 
@@ -159,6 +159,23 @@ int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const w
                       int B, int C, int N, int K, int levels,
                       int dtype, int param_dtype,
                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- the passes of a WTConvNeXt block around its WTConv layer, each as one kernel that transposes through LDS.
+ * Forward only (inference); activations in `dtype`, weight / bias / gamma in `param_dtype`; C must be even.
+ *
+ * wtconv_channel_norm: LayerNorm over the channels of every pixel of x (B, C, HW), biased variance, `eps` inside
+ * the square root.  out_nhwc != 0 writes (B, HW, C): the permute to NHWC followed by nn.LayerNorm that the block
+ * does after conv_dw (wtconvnext/wtconvnext.py:132-133).  out_nhwc == 0 writes (B, C, HW): the LayerNorm2d of the
+ * stem and of the downsample layers (wtconvnext/wtconvnext.py:171, 296).  x and out must not overlap. */
+int wtconv_channel_norm(const void* x, void* out, const void* weight, const void* bias, int B, int C, int HW,
+                        float eps, int dtype, int param_dtype, int out_nhwc, void* stream);
+
+/* wtconv_block_residual: out (B, C, HW) = shortcut (B, C, HW) + gamma[c] * y, with y (B, HW, C) the NHWC output
+ * of the block's MLP: the permute back to NCHW, the layer scale and the residual add of
+ * wtconvnext/wtconvnext.py:135-140 (drop_path is the identity at inference).  gamma may be NULL (no layer
+ * scale).  out may be the shortcut itself. */
+int wtconv_block_residual(const void* y, const void* shortcut, const void* gamma, void* out, int B, int C, int HW,
+                          int dtype, int param_dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -8,7 +8,7 @@ from . import _build
 MAX_LEVELS = 5
 F32, BF16 = 0, 1
 PASS_FORWARD, PASS_BACKWARD_INPUT, PASS_BACKWARD_PARAMS, PASS_BACKWARD = 0, 1, 2, 3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Params(ctypes.Structure):
@@ -43,6 +43,9 @@ for _name in ("wtconv1d_forward", "wtconv1d_backward_input"):
     EXPORTS[_name] = (_i, [_p, _p, ctypes.POINTER(Params)] + [_i] * 7 + [_p, _z, _p])
 EXPORTS["wtconv1d_backward_params"] = (
     _i, [_p, _p, ctypes.POINTER(Params), ctypes.POINTER(ParamGrads)] + [_i] * 7 + [_p, _z, _p])
+_f = ctypes.c_float
+EXPORTS["wtconv_channel_norm"] = (_i, [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _i, _p])
+EXPORTS["wtconv_block_residual"] = (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p])
 
 _lib = None
 _lock = threading.Lock()

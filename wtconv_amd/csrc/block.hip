@@ -1,0 +1,135 @@
+// Host side of the block-epilogue kernels (kernels_block.h): argument checks, tile choice, launches.
+// Allocates nothing, never synchronises.
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "common.h"
+#include "host_util.h"
+#include "kernels_block.h"
+
+namespace wt {
+namespace {
+
+// Largest power-of-two pixel tile (8..64) whose [C][tp + 1] floats, plus the per-pixel statistics, stay within
+// 48 KB of LDS (three workgroups per CU); false if even 8 pixels do not fit or the sizes overflow the indexing.
+bool make_block_tile(int C, int HW, BlockTile* out, size_t* lds_bytes) {
+  BlockTile t = {};
+  t.C = C; t.HW = HW;
+  int tp = 64;
+  // tile, two sets of partial sums [256 / p][p], mean and rstd [2][p], weight and bias [2][C]
+  auto bytes = [&](int p) { return (static_cast<size_t>(C) * (p + 1) + 2 * kBlockThreads + 2 * p + 2 * static_cast<size_t>(C)) * sizeof(float); };
+  while (tp > 8 && bytes(tp) > 48 * 1024) tp >>= 1;
+  if (bytes(tp) > kLdsLimitBytes) return false;
+  while (tp > 8 && tp / 2 >= HW) tp >>= 1;          // tiny images: no lanes without a pixel
+  t.tp = tp;
+  t.tp_shift = 0;
+  while ((1 << t.tp_shift) < tp) ++t.tp_shift;
+  t.tiles = (HW + tp - 1) / tp;
+  // reciprocal of C, exact for every dividend below tp * C (checked)
+  const unsigned long long m = ((1ull << 32) + C - 1) / C;
+  if (m >= (1ull << 32)) return false;
+  t.mg_c = static_cast<unsigned>(m);
+  for (int v = 0; v < tp * C; v += 1)
+    if (static_cast<int>((static_cast<unsigned long long>(v) * t.mg_c) >> 32) != v / C) return false;
+  *out = t;
+  *lds_bytes = bytes(tp);
+  return true;
+}
+
+struct TileKey {
+  int C, HW;
+  bool operator==(const TileKey& o) const { return C == o.C && HW == o.HW; }
+};
+struct TileKeyHash {
+  size_t operator()(const TileKey& k) const { return (static_cast<size_t>(k.C) << 32) ^ static_cast<size_t>(k.HW); }
+};
+struct TileVal { bool ok; BlockTile t; size_t lds; };
+
+const TileVal& block_tile_cached(int C, int HW) {
+  static thread_local std::unordered_map<TileKey, TileVal, TileKeyHash> cache;
+  const TileKey key = {C, HW};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    if (cache.size() > 4096) cache.clear();
+    TileVal v = {};
+    v.ok = make_block_tile(C, HW, &v.t, &v.lds);
+    it = cache.emplace(key, v).first;
+  }
+  return it->second;
+}
+
+int check_block_args(const char* fn, int B, int C, int HW, int dtype, int pdtype, const TileVal** tv) {
+  if (B <= 0 || C <= 0 || HW <= 0) return fail(WTCONV_E_ARG, "%s: sizes must be positive (got B=%d C=%d HW=%d)", fn, B, C, HW);
+  if (C % 2) return fail(WTCONV_E_UNSUPPORTED, "%s: the channel count must be even (got %d)", fn, C);
+  if ((dtype != WTCONV_F32 && dtype != WTCONV_BF16) || (pdtype != WTCONV_F32 && pdtype != WTCONV_BF16))
+    return fail(WTCONV_E_ARG, "%s: unknown dtype code", fn);
+  if (B > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: batch %d exceeds the launch grid", fn, B);
+  if (static_cast<long long>(C) * HW > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "%s: an image of %d x %d elements is too large", fn, C, HW);
+  const TileVal& v = block_tile_cached(C, HW);
+  if (!v.ok) return fail(WTCONV_E_UNSUPPORTED, "%s: %d channels do not fit a tile in LDS", fn, C);
+  *tv = &v;
+  return 0;
+}
+
+}  // namespace
+}  // namespace wt
+
+using namespace wt;
+
+extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight, const void* bias, int B, int C, int HW,
+                                   float eps, int dtype, int param_dtype, int out_nhwc, void* stream_) {
+  const char* fn = "wtconv_channel_norm";
+  const TileVal* tv = nullptr;
+  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv)) return e;
+  if (x == nullptr || out == nullptr || weight == nullptr || bias == nullptr) return fail(WTCONV_E_ARG, "%s: null pointer", fn);
+  if (x == out) return fail(WTCONV_E_ARG, "%s: in-place use is not supported (tiles of the output overlap other tiles' input)", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % (2 * esz)))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned (input to one element, output to two)", fn);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const dim3 grid(tv->t.tiles, B);
+  // rows of whole aligned 4-element vectors move as such
+  const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0;
+  auto launch = [&](auto kern, auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (int e = allow_lds(kern, tv->lds)) return e;
+    WT_LAUNCH(kern, grid, dim3(kBlockThreads), tv->lds, stream, static_cast<const T*>(x), static_cast<T*>(out),
+              weight, bias, param_dtype, eps, out_nhwc, tv->t);
+    return check_launch("channel_norm_kernel");
+  };
+  if (dtype == WTCONV_F32)
+    return vec ? launch(channel_norm_kernel<float, true>, static_cast<float*>(nullptr))
+               : launch(channel_norm_kernel<float, false>, static_cast<float*>(nullptr));
+  return vec ? launch(channel_norm_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
+             : launch(channel_norm_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+}
+
+extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const void* gamma, void* out, int B, int C,
+                                     int HW, int dtype, int param_dtype, void* stream_) {
+  const char* fn = "wtconv_block_residual";
+  const TileVal* tv = nullptr;
+  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv)) return e;
+  if (y == nullptr || shortcut == nullptr || out == nullptr) return fail(WTCONV_E_ARG, "%s: null pointer", fn);
+  if (y == out) return fail(WTCONV_E_ARG, "%s: the output may alias the shortcut, not the NHWC input", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(y) % (2 * esz)) || (reinterpret_cast<uintptr_t>(shortcut) % esz) ||
+      (reinterpret_cast<uintptr_t>(out) % esz))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned (NHWC input to two elements, the others to one)", fn);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const dim3 grid(tv->t.tiles, B);
+  const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(shortcut) % (4 * esz) == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0;
+  auto launch = [&](auto kern, auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (int e = allow_lds(kern, tv->lds)) return e;
+    WT_LAUNCH(kern, grid, dim3(kBlockThreads), tv->lds, stream, static_cast<const T*>(y), static_cast<const T*>(shortcut),
+              gamma, param_dtype, static_cast<T*>(out), tv->t);
+    return check_launch("block_residual_kernel");
+  };
+  if (dtype == WTCONV_F32)
+    return vec ? launch(block_residual_kernel<float, true>, static_cast<float*>(nullptr))
+               : launch(block_residual_kernel<float, false>, static_cast<float*>(nullptr));
+  return vec ? launch(block_residual_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
+             : launch(block_residual_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+}

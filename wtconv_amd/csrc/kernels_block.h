@@ -1,0 +1,234 @@
+// What a WTConvNeXt block does around its WTConv layer (wtconvnext/wtconvnext.py:125-140 of the reference): after
+// `conv_dw` the activations are permuted to NHWC and LayerNorm-ed over the channels (:132-133); after the MLP they
+// are permuted back, scaled per channel and added to the shortcut (:135-140).  As separate passes these are four
+// trips through HBM, two of them layout copies; here each side is one kernel that transposes through LDS:
+//   channel_norm_kernel    NCHW -> LayerNorm over C -> NHWC (or NCHW: the LayerNorm2d of stem and downsample layers)
+//   block_residual_kernel  NHWC y, NCHW shortcut -> shortcut + gamma[c] * y, NCHW
+// A workgroup takes a tile of TP consecutive pixels of one image with all their channels: [C][TP + 1] floats in
+// LDS (the odd row pitch keeps both the pixel-major and the channel-major sweep free of bank conflicts).  The
+// NCHW side moves TP contiguous elements per channel, the NHWC side the tile's TP * C elements, which are one
+// contiguous run.  Statistics are two sweeps over LDS in fp32 (mean, then the sum of squared deviations).
+#pragma once
+
+#include "common.h"
+
+namespace wt {
+
+constexpr int kBlockThreads = 256;
+
+struct BlockTile {
+  int C, HW;
+  int tp;            // pixels per tile: a power of two, 8..64
+  int tp_shift;
+  int tiles;         // tiles per image
+  unsigned mg_c;     // reciprocal of C for dividends < tp * C (shift 32)
+};
+
+__device__ __forceinline__ int div_c(int v, unsigned magic) {
+#ifdef WT_EMULATE
+  return static_cast<int>((static_cast<unsigned long long>(static_cast<unsigned>(v)) * magic) >> 32);
+#else
+  return static_cast<int>(__umulhi(static_cast<unsigned>(v), magic));
+#endif
+}
+
+template <typename T>
+__device__ __forceinline__ void store_pair(T* p, float a, float b);
+template <> __device__ __forceinline__ void store_pair<float>(float* p, float a, float b) {
+  *reinterpret_cast<float2*>(p) = make_float2(a, b);
+}
+template <> __device__ __forceinline__ void store_pair<bf16_t>(bf16_t* p, float a, float b) {
+  *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(a, b);
+}
+template <typename T>
+__device__ __forceinline__ void load_pair(const T* p, float& a, float& b);
+template <> __device__ __forceinline__ void load_pair<float>(const float* p, float& a, float& b) {
+  const float2 v = *reinterpret_cast<const float2*>(p);
+  a = v.x; b = v.y;
+}
+template <> __device__ __forceinline__ void load_pair<bf16_t>(const bf16_t* p, float& a, float& b) {
+  const uint32_t v = *reinterpret_cast<const uint32_t*>(p);
+  a = __uint_as_float(v << 16); b = __uint_as_float(v & 0xffff0000u);
+}
+
+// four consecutive elements at an address aligned to four elements
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  float4 v;
+  __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
+  __device__ __forceinline__ void get(float (&f)[4]) const { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
+};
+template <> struct Quad<bf16_t> {
+  uint2 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const uint2*>(p); }
+  __device__ __forceinline__ void get(float (&f)[4]) const {
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+};
+
+constexpr int kQuadBatch = 6;      // vector loads a thread keeps in flight before it writes them to LDS
+
+// NCHW tile -> LDS [C][tp + 1]; pixels past the image are left alone (never read back).
+// VEC: HW is a multiple of 4 and the tensor 4-element aligned, so rows move as 4-element vectors.
+template <typename T, bool VEC>
+__device__ __forceinline__ void tile_from_nchw(const T* __restrict__ img, float* lds, const BlockTile& t, int p0, int tid) {
+  const int pitch = t.tp + 1;
+  if constexpr (VEC) {
+    const int gshift = t.tp_shift - 2;                       // 4-pixel groups per tile row
+    const int g = tid & ((1 << gshift) - 1), c0 = tid >> gshift, cstep = kBlockThreads >> gshift;
+    const int p = 4 * g;
+    if (p0 + p < t.HW) {                                     // (HW % 4 == 0: a group is inside the image or outside)
+      const T* src = img + p0 + p;
+      for (int cb = c0; cb < t.C; cb += kQuadBatch * cstep) {
+        Quad<T> q[kQuadBatch];
+#pragma unroll
+        for (int k = 0; k < kQuadBatch; ++k) {
+          const int c = cb + k * cstep;
+          if (c < t.C) q[k].load(src + static_cast<size_t>(c) * t.HW);
+        }
+#pragma unroll
+        for (int k = 0; k < kQuadBatch; ++k) {
+          const int c = cb + k * cstep;
+          if (c < t.C) {
+            float f[4];
+            q[k].get(f);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) lds[c * pitch + p + j] = f[j];
+          }
+        }
+      }
+    }
+  } else {
+    const int p = tid & (t.tp - 1), c0 = tid >> t.tp_shift, cstep = kBlockThreads >> t.tp_shift;
+    if (p0 + p < t.HW)
+      for (int c = c0; c < t.C; c += cstep) lds[c * pitch + p] = to_f32<T>(img[static_cast<size_t>(c) * t.HW + p0 + p]);
+  }
+}
+
+// Grid (tiles, B).  out_nhwc != 0: out is (B, HW, C); else (B, C, HW).
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlockThreads)
+channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __restrict__ weight,
+                    const void* __restrict__ bias, int pdtype, float eps, int out_nhwc, const BlockTile t) {
+  WT_SHARED_FLOATS(lds);
+  const int tid = threadIdx.x;
+  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  const int pitch = t.tp + 1, C = t.C;
+  const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
+  float* psum = lds + C * pitch;                 // [parts][tp] partial sums
+  float* pvar = psum + kBlockThreads;            // [parts][tp] partial sums of squared deviations
+  float* stat = pvar + kBlockThreads;            // mean[tp], rstd[tp]
+  float* wgt = stat + 2 * t.tp;                  // weight[C], bias[C]
+  const T* img = x + static_cast<size_t>(b) * C * t.HW;
+  tile_from_nchw<T, VEC>(img, lds, t, p0, tid);
+  for (int c = tid; c < C; c += kBlockThreads) {
+    wgt[c] = load_param(weight, pdtype, c);
+    wgt[C + c] = load_param(bias, pdtype, c);
+  }
+  __syncthreads();
+  const int p = tid & (t.tp - 1), part_i = tid >> t.tp_shift, parts = kBlockThreads >> t.tp_shift;
+  const bool live = p < np;
+  float s = 0.f;
+  if (live)
+    for (int c = part_i; c < C; c += parts) s += lds[c * pitch + p];
+  psum[part_i * t.tp + p] = s;
+  __syncthreads();
+  float mean = 0.f;
+  for (int k = 0; k < parts; ++k) mean += psum[k * t.tp + p];
+  mean *= 1.f / static_cast<float>(C);
+  float v = 0.f;
+  if (live)
+    for (int c = part_i; c < C; c += parts) {
+      const float d = lds[c * pitch + p] - mean;
+      v += d * d;
+    }
+  pvar[part_i * t.tp + p] = v;
+  __syncthreads();
+  float var = 0.f;
+  for (int k = 0; k < parts; ++k) var += pvar[k * t.tp + p];
+  const float rstd = 1.f / sqrtf(var * (1.f / static_cast<float>(C)) + eps);
+  if (out_nhwc) {
+    if (part_i == 0) { stat[p] = mean; stat[t.tp + p] = rstd; }
+    __syncthreads();
+    // the tile's output is one contiguous run of np * C elements; C is even, so pairs never straddle a pixel
+    T* dst = out + (static_cast<size_t>(b) * t.HW + p0) * C;
+    const int npair = (np * C) >> 1;
+    for (int i = tid; i < npair; i += kBlockThreads) {
+      const int e = 2 * i;
+      const int pp = div_c(e, t.mg_c), c = e - pp * C;
+      const float m = stat[pp], r = stat[t.tp + pp];
+      const float a = (lds[c * pitch + pp] - m) * r * wgt[c] + wgt[C + c];
+      const float bb = (lds[(c + 1) * pitch + pp] - m) * r * wgt[c + 1] + wgt[C + c + 1];
+      store_pair<T>(dst + e, a, bb);
+    }
+  } else {
+    T* dst = out + static_cast<size_t>(b) * C * t.HW + p0;
+    if (live)
+      for (int c = part_i; c < C; c += parts)
+        dst[static_cast<size_t>(c) * t.HW + p] = from_f32<T>((lds[c * pitch + p] - mean) * rstd * wgt[c] + wgt[C + c]);
+  }
+}
+
+// Grid (tiles, B).  y is (B, HW, C); shortcut and out are (B, C, HW); gamma may be null (no layer scale).
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlockThreads)
+block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, const void* __restrict__ gamma,
+                      int pdtype, T* __restrict__ out, const BlockTile t) {
+  WT_SHARED_FLOATS(lds);
+  const int tid = threadIdx.x;
+  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  const int pitch = t.tp + 1, C = t.C;
+  const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
+  const T* src = y + (static_cast<size_t>(b) * t.HW + p0) * C;
+  const int npair = (np * C) >> 1;
+  for (int i = tid; i < npair; i += kBlockThreads) {
+    const int e = 2 * i;
+    const int pp = div_c(e, t.mg_c), c = e - pp * C;
+    float a, bb;
+    load_pair<T>(src + e, a, bb);
+    lds[c * pitch + pp] = a;
+    lds[(c + 1) * pitch + pp] = bb;
+  }
+  __syncthreads();
+  if constexpr (VEC) {
+    const int gshift = t.tp_shift - 2;
+    const int g = tid & ((1 << gshift) - 1), c0 = tid >> gshift, cstep = kBlockThreads >> gshift;
+    const int p = 4 * g;
+    if (p < np) {
+      const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + p;
+      for (int cb = c0; cb < C; cb += kQuadBatch * cstep) {
+        Quad<T> q[kQuadBatch];
+#pragma unroll
+        for (int k = 0; k < kQuadBatch; ++k) {
+          const int c = cb + k * cstep;
+          if (c < C) q[k].load(shortcut + base + static_cast<size_t>(c) * t.HW);
+        }
+#pragma unroll
+        for (int k = 0; k < kQuadBatch; ++k) {
+          const int c = cb + k * cstep;
+          if (c < C) {
+            const float gm = gamma != nullptr ? load_param(gamma, pdtype, c) : 1.f;
+            float f[4];
+            q[k].get(f);
+            T* o = out + base + static_cast<size_t>(c) * t.HW;
+            store_pair<T>(o, f[0] + gm * lds[c * pitch + p], f[1] + gm * lds[c * pitch + p + 1]);
+            store_pair<T>(o + 2, f[2] + gm * lds[c * pitch + p + 2], f[3] + gm * lds[c * pitch + p + 3]);
+          }
+        }
+      }
+    }
+  } else {
+    const int p = tid & (t.tp - 1), c0 = tid >> t.tp_shift, cstep = kBlockThreads >> t.tp_shift;
+    if (p < np) {
+      const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + p;
+      for (int c = c0; c < C; c += cstep) {
+        const float g = gamma != nullptr ? load_param(gamma, pdtype, c) : 1.f;
+        const size_t o = base + static_cast<size_t>(c) * t.HW;
+        out[o] = from_f32<T>(to_f32<T>(shortcut[o]) + g * lds[c * pitch + p]);
+      }
+    }
+  }
+}
+
+}  // namespace wt

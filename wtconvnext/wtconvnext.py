@@ -21,6 +21,15 @@ import torch.nn.functional as F
 from wtconv import WTConv2d
 
 
+def _block_ops():
+    """The fused block passes of the HIP library, or None where it is not importable (CPU-only use of the harness)."""
+    try:
+        from wtconv_amd import block_ops
+        return block_ops
+    except ImportError:
+        return None
+
+
 class LayerNorm2d(nn.LayerNorm):
     """LayerNorm over the channel dimension of an NCHW tensor."""
 
@@ -28,6 +37,9 @@ class LayerNorm2d(nn.LayerNorm):
         super().__init__(num_channels, eps=eps)
 
     def forward(self, x):
+        ops = _block_ops()
+        if ops is not None and self.elementwise_affine and self.bias is not None and ops.usable(x, self.weight, self.bias):
+            return ops.channel_norm(x, self.weight, self.bias, self.eps, nhwc=False)      # inference: one kernel
         x = x.permute(0, 2, 3, 1)
         x = F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps)
         return x.permute(0, 3, 1, 2)
@@ -76,6 +88,16 @@ class WTConvNeXtBlock(nn.Module):
     def forward(self, x):
         shortcut = x
         x = self.conv_dw(x)
+        ops = _block_ops()
+        drops = self.training and not isinstance(self.drop_path, nn.Identity)
+        if (ops is not None and not drops and x.is_contiguous() and shortcut.is_contiguous()
+                and ops.usable(x, self.norm.weight, self.norm.bias, self.gamma)
+                and ops.usable(shortcut)):
+            # inference on the GPU: NCHW -> LayerNorm -> NHWC, and NHWC -> layer scale -> + shortcut -> NCHW, are one
+            # kernel each instead of a layout copy plus an elementwise pass each
+            x = ops.channel_norm(x, self.norm.weight, self.norm.bias, self.norm.eps, nhwc=True)
+            x = self.mlp(x)
+            return ops.block_residual(x.contiguous(), shortcut, self.gamma)
         x = x.permute(0, 2, 3, 1)
         x = self.mlp(self.norm(x))
         x = x.permute(0, 3, 1, 2)
