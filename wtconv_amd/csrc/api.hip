@@ -51,10 +51,10 @@ static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float
 }
 
 // ---- 2-D dispatch over (dtype, K, level-1 strip width) -------------------------------
-template <typename T, int K, int TJ1, int MODE>
+template <typename T, int K, int TJ1, int MODE, typename Geo = PlaneGeoRuntime>
 static int run_plane2d_mode(const void* x, void* out, const float* fw, const float* fb, const Plan2D& pl,
                             hipStream_t stream) {
-  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC, MODE>;
+  auto kern = wt2d_plane_kernel<T, K, TJ1, kTJC, MODE, Geo>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   const int sg = 1 << pl.sg_shift;
@@ -64,6 +64,27 @@ static int run_plane2d_mode(const void* x, void* out, const float* fw, const flo
   if (nwg > nunits) nwg = nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(pl.block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), fw, fb, pl);
   return check_launch("wt2d_plane_kernel");
+}
+
+// Plane shapes of the WTConvNeXt stages with K = 5: geometry as a compile-time constant.  Returns 1 if the shape
+// is not one of them (or the run-time plan differs, e.g. unaligned pointers), else the launch's result.
+template <typename T>
+static int run_plane2d_static(int K, int tj1, const void* x, void* out, const float* fw, const float* fb,
+                              const Plan2D& pl, hipStream_t stream) {
+#ifndef WT_EMULATE
+  if (K != 5 || pl.H != pl.W) return 1;
+#define WT_TRY(H_, L_)                                                                                  \
+  if (pl.H == H_ && pl.L == L_) {                                                                       \
+    using G = PlaneGeoStatic<H_, H_, 5, L_>;                                                            \
+    constexpr Plan2D g = G::plan();                                                                     \
+    if (tj1 == G::tj1() && same_plane_geometry(g, pl))                                                  \
+      return run_plane2d_mode<T, 5, G::tj1(), G::mode(), G>(x, out, fw, fb, pl, stream);                \
+    return 1;                                                                                           \
+  }
+  WT_TRY(56, 3) WT_TRY(28, 3) WT_TRY(14, 2) WT_TRY(7, 2)
+#undef WT_TRY
+#endif
+  return 1;
 }
 
 template <typename T, int K, int TJ1>
@@ -97,15 +118,37 @@ static int run_plane2d_k(int K, int tj1, const void* x, void* out, const float* 
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
 
-template <typename T, int K, int L>
+template <typename T, int K, int L, typename Geo = PlaneGeoRuntime>
 static int run_wgrad2d(const void* x, const void* g, float* partial, const Plan2D& pl, int B, int bchunk,
                        int nchunk, hipStream_t stream) {
-  auto kern = wt2d_wgrad_kernel<T, K, L, kTJW>;
+  auto kern = wt2d_wgrad_kernel<T, K, L, kTJW, Geo>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(512), lds, stream, static_cast<const T*>(x), static_cast<const T*>(g),
             partial, pl, B, bchunk);
   return check_launch("wt2d_wgrad_kernel");
+}
+
+// Plane shapes of the WTConvNeXt stages with K = 5 at their usual planes per iteration: geometry as a compile-time
+// constant.  Returns 1 if the launch is not one of them, else the launch's result.
+template <typename T>
+static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
+                              int bchunk, int nchunk, hipStream_t stream) {
+#ifndef WT_EMULATE
+  if (K != 5 || pl.H != pl.W) return 1;
+#define WT_TRY(H_, L_)                                                                                   \
+  if (pl.H == H_ && L == L_) {                                                                           \
+    constexpr int PB = wgrad_planes_per_iter(128, H_, H_, 5, L_);                                        \
+    using G = WgradGeoStatic<H_, H_, 5, L_, PB>;                                                         \
+    constexpr Plan2D gp = G::plan();                                                                     \
+    if (same_wgrad_geometry(gp, pl))                                                                     \
+      return run_wgrad2d<T, 5, L_, G>(x, g, partial, pl, B, bchunk, nchunk, stream);                     \
+    return 1;                                                                                            \
+  }
+  WT_TRY(56, 3) WT_TRY(28, 3) WT_TRY(14, 2) WT_TRY(7, 2)
+#undef WT_TRY
+#endif
+  return 1;
 }
 
 template <typename T, int K>
@@ -342,6 +385,10 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
+  if (dtype == WTCONV_F32) {
+    const int e = run_plane2d_static<float>(K, tj1, x, out, fw, fb, pl, stream);
+    if (e != 1) return e;
+  }
   return dtype == WTCONV_F32 ? run_plane2d_k<float>(K, tj1, x, out, fw, fb, pl, stream)
                              : run_plane2d_k<bf16_t>(K, tj1, x, out, fw, fb, pl, stream);
 }
@@ -693,8 +740,10 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
     Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
     finish_wgrad_plan(&pl, K);
     wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
-    e = dtype == WTCONV_F32 ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
-                            : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
+    e = dtype == WTCONV_F32 ? run_wgrad2d_static<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream) : 1;
+    if (e == 1)
+      e = dtype == WTCONV_F32 ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+                              : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
   } else {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     nchunk = stream_chunks(B, C, H, W);

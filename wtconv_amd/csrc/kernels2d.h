@@ -635,11 +635,17 @@ __device__ __forceinline__ void zero_lds(float* lds, int nfloats) {
 // with levels 2-3 produced at the commit, 1: fused vector load without prefetch, 2: element-wise
 // load), so that the hot variant does not carry
 // the registers of the others.
-template <typename T, int K, int TJ1, int TJC, int MODE>
+// Geo: the plan's geometry as a compile-time constant for the common shapes (LDS offsets and strides fold into
+// instruction immediates, loops over levels unroll), or the run-time plan of the argument for any other shape;
+// batch, channels and what follows from them always come from the argument.
+template <typename T, int K, int TJ1, int TJC, int MODE, typename Geo>
 __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                          const float* __restrict__ fw,
-                                                         const float* __restrict__ fb, Plan2D pl) {
+                                                         const float* __restrict__ fb, const Plan2D plarg) {
   WT_SHARED_FLOATS(lds_all);
+  static constexpr Plan2D kGeo = Geo::plan();
+  const Plan2D& pl = Geo::kStatic ? kGeo : plarg;
+  const int nB = plarg.B, nC = plarg.C, nplanes = plarg.nplanes, gpc = plarg.groups_per_channel;
   constexpr int KK = K * K;
   const int NF = 1 + 4 * pl.L;
   const size_t plane_elems = static_cast<size_t>(pl.H) * pl.W;
@@ -651,7 +657,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   float* lds = lds_all + slot * pl.plane_lds_floats;
   const int wave = tid >> 6;
   const int ppw = sg < kWave ? kWave >> pl.sg_shift : 1;      // planes per wave
-  const int nunits = sg < kWave ? (pl.C * pl.groups_per_channel + 3) / 4 : (pl.nplanes + slots - 1) / slots;
+  const int nunits = sg < kWave ? (nC * gpc + 3) / 4 : (nplanes + slots - 1) / slots;
 
   // Plane of this thread in a work unit (-1: none) and its (wave-uniform) channel.  The
   // divisions happen once: `locate` positions the state on the workgroup's first unit, and
@@ -661,28 +667,28 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
   const int G = gridDim.x;
   int step_c = 0, step_q = 0, step_r = 0;
   if (sg < kWave) {
-    step_q = (4 * G) / pl.groups_per_channel;
-    step_r = 4 * G - step_q * pl.groups_per_channel;
+    step_q = (4 * G) / gpc;
+    step_r = 4 * G - step_q * gpc;
   } else {
-    step_c = static_cast<int>((static_cast<long long>(G) * slots) % pl.C);
+    step_c = static_cast<int>((static_cast<long long>(G) * slots) % nC);
   }
   auto resolve = [&](Loc& s) {
     if (sg < kWave) {
       const int b = imul(s.rem, ppw) + ((tid & (kWave - 1)) >> pl.sg_shift);
-      s.plane = (s.c < pl.C && b < pl.B) ? imul(b, pl.C) + s.c : -1;
+      s.plane = (s.c < nC && b < nB) ? imul(b, nC) + s.c : -1;
     } else {
-      s.plane = s.key < pl.nplanes ? s.key : -1;
+      s.plane = s.key < nplanes ? s.key : -1;
     }
   };
   auto locate = [&](int u, Loc& s) {
     if (sg < kWave) {
       const int gidx = u * 4 + wave;
-      s.c = gidx / pl.groups_per_channel;
-      s.rem = gidx - s.c * pl.groups_per_channel;
+      s.c = gidx / gpc;
+      s.rem = gidx - s.c * gpc;
       s.key = 0;
     } else {
       s.key = u * slots + slot;
-      s.c = s.key % pl.C;
+      s.c = s.key % nC;
       s.rem = 0;
     }
     resolve(s);
@@ -691,16 +697,16 @@ __global__ __launch_bounds__(512, 4) void wt2d_plane_kernel(const T* __restrict_
     if (sg < kWave) {
       s.c += step_q;
       s.rem += step_r;
-      if (s.rem >= pl.groups_per_channel) { s.rem -= pl.groups_per_channel; s.c += 1; }
+      if (s.rem >= gpc) { s.rem -= gpc; s.c += 1; }
     } else {
       s.key += G * slots;           // may pass nplanes: resolve() maps that to "no plane"
       s.c += step_c;
-      if (s.c >= pl.C) s.c -= pl.C;
+      if (s.c >= nC) s.c -= nC;
     }
     resolve(s);
   };
   // the channel used for the weights (clamped: a thread without a plane still runs uniform code)
-  auto channel_of = [&](const Loc& s) { return s.c < pl.C ? s.c : pl.C - 1; };
+  auto channel_of = [&](const Loc& s) { return s.c < nC ? s.c : nC - 1; };
 
   constexpr bool kPrefetch = MODE == 0 || MODE == 3;
   float fa[kFetchPasses][4], fbuf[kFetchPasses][4];
@@ -877,11 +883,14 @@ __device__ __forceinline__ void corr_level(const float* __restrict__ A, int astr
 constexpr int wgrad_sets(int L) { return L >= 4 ? 3 : (L >= 2 ? 2 : 1); }
 constexpr int kStripMinWidth = 12;   // coarse levels of the weight-gradient kernel: strips from this width on
 
-template <typename T, int K, int L, int TJ>
+template <typename T, int K, int L, int TJ, typename Geo>
 __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ g,
-                                                         float* __restrict__ partial, Plan2D pl,
+                                                         float* __restrict__ partial, const Plan2D plarg,
                                                          int B, int bchunk) {
   WT_SHARED_FLOATS(lds);
+  static constexpr Plan2D kGeo = Geo::plan();      // compile-time geometry for the common shapes (see wt2d_plane_kernel)
+  const Plan2D& pl = Geo::kStatic ? kGeo : plarg;
+  const int nC = plarg.C;
   constexpr int KK = K * K;
   constexpr int R = K / 2;
   constexpr int NF = 1 + 4 * L;
@@ -927,7 +936,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
   float xa[1][4], xb[1][4], ga[1][4], gb[1][4];
   if (pl.prefetch && has_slot) {
     const bool valid = b_begin + slot < b_end;
-    const size_t off = (static_cast<size_t>(valid ? b_begin + slot : b_begin) * pl.C + c) * plane_elems;
+    const size_t off = (static_cast<size_t>(valid ? b_begin + slot : b_begin) * nC + c) * plane_elems;
     plane_fetch<T, 1>(x + off, pl.H, pl.W, ltid, nps, xa, xb);
     plane_fetch<T, 1>(g + off, pl.H, pl.W, ltid, nps, ga, gb);
   }
@@ -940,7 +949,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     WT_LAUNDER_LANE_INT(ltid);
     WT_LAUNDER_LANE_INT(lane);
     const bool valid = has_slot && b0 + slot < b_end;
-    const size_t plane_off = (static_cast<size_t>(valid ? b0 + slot : b0) * pl.C + c) * plane_elems;
+    const size_t plane_off = (static_cast<size_t>(valid ? b0 + slot : b0) * nC + c) * plane_elems;
     int l0 = 2;
     WT_WAVE_PRIORITY(3);
     if (pl.prefetch && pl.fuse >= 2) {      // one plane per iteration: every lane takes part
@@ -975,7 +984,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     WT_LDS_BARRIER();
     if (pl.prefetch && has_slot && b0 + pb < b_end) {
       const bool nvalid = b0 + pb + slot < b_end;
-      const size_t off = (static_cast<size_t>(nvalid ? b0 + pb + slot : b0) * pl.C + c) * plane_elems;
+      const size_t off = (static_cast<size_t>(nvalid ? b0 + pb + slot : b0) * nC + c) * plane_elems;
       plane_fetch<T, 1>(x + off, pl.H, pl.W, ltid, nps, xa, xb);   // an absent plane re-reads plane b0:
       plane_fetch<T, 1>(g + off, pl.H, pl.W, ltid, nps, ga, gb);   //   zeroed at commit
     }
@@ -1043,7 +1052,7 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
     if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
   WT_LDS_BARRIER();
-  float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * (NF * KK + 1);
+  float* dst = partial + (static_cast<size_t>(chunk) * nC + c) * (NF * KK + 1);
   for (int o = tid; o < NF * KK + 1; o += blockDim.x) {
     float v = 0.f;
     if (o == NF * KK) {

@@ -10,15 +10,15 @@
 
 namespace wt {
 
-inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Strip widths of the 2-D kernels (outputs per work item along a row).
 constexpr int kTJC = 1;     // coarser levels of the plane kernel: single coefficients keep the most lanes busy
                             // (measured against strips of 2: 28x28 planes 106 -> 100 us, 14x14 73 -> 71, 56x56 equal)
 constexpr int kTJW = 4;     // weight-gradient correlation strips
 
-inline int pow2_ceil(int v) { int p = 1; while (p < v) p *= 2; return p; }
-inline int log2_int(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
+constexpr int pow2_ceil(int v) { int p = 1; while (p < v) p *= 2; return p; }
+constexpr int log2_int(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
 
 // Level-1 strip width and threads per plane of the plane kernel: the pair that keeps most
 // lanes busy in the level-1 phase (ties: the wider strip, which reads less LDS per FMA),
@@ -26,7 +26,7 @@ inline int log2_int(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
 // `plane_lds_bytes` each) leave room for fewer than three workgroups per CU: with two, the
 // phases of a plane are latency bound (measured on 14x14 planes: 88 -> 76 us with 32 instead
 // of 16 threads per plane, i.e. half the slots).
-inline void choose_plane_shape(int h1, int w1, size_t plane_lds_bytes, int* tj1, int* sg_shift) {
+constexpr void choose_plane_shape(int h1, int w1, size_t plane_lds_bytes, int* tj1, int* sg_shift) {
   double best = -1.0;
   for (int tj = 4; tj >= 1; tj /= 2) {
     const int gs = pow2_ceil((w1 + tj - 1) / tj);
@@ -48,8 +48,8 @@ inline void choose_plane_shape(int h1, int w1, size_t plane_lds_bytes, int* tj1,
 // P zero rows that serves as bottom halo of the upper and top halo of the lower plane.
 // with_grad_pyramid adds the padded pyramid of grad_out used by the weight-gradient kernel
 // (and drops the Z buffers it does not need).
-inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
-                          size_t elem_size, const void* p0, const void* p1, const void* p2, int pb = 1) {
+constexpr Plan2D make_plan2d_geometry(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
+                                      int pb) {
   Plan2D pl = {};
   pl.B = B; pl.C = C; pl.H = H; pl.W = W; pl.L = L;
   pl.nplanes = B * C;
@@ -87,6 +87,13 @@ inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_gr
   pl.slot_shift = log2_int(nthreads);
   pl.lds_floats = pl.plane_lds_floats;
   pl.groups_per_channel = 1;
+  pl.vec_ok = W % 4 == 0;                         // (and aligned pointers: make_plan2d)
+  return pl;
+}
+
+inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_grad_pyramid, int nthreads,
+                          size_t elem_size, const void* p0, const void* p1, const void* p2, int pb = 1) {
+  Plan2D pl = make_plan2d_geometry(B, C, H, W, K, L, with_grad_pyramid, nthreads, pb);
   const uintptr_t mask = 4 * elem_size - 1;       // 4-element vectors: 16 B (fp32) / 8 B (bf16)
   auto aligned = [mask](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
   pl.vec_ok = (W % 4 == 0) && aligned(p0) && aligned(p1) && aligned(p2);
@@ -94,7 +101,7 @@ inline Plan2D make_plan2d(int B, int C, int H, int W, int K, int L, bool with_gr
 }
 
 // Completes a plan for the plane kernel: threads per plane, slots per workgroup, prefetch.
-inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
+constexpr void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
   pl->sg_shift = tj1_sg_shift;
   const int sg = 1 << pl->sg_shift;
   pl->block = 256;   // (two whole planes per 512-thread workgroup measured slower: lockstep phases)
@@ -112,16 +119,54 @@ inline void finish_plane_plan(Plan2D* pl, int tj1_sg_shift) {
   }
 }
 
+// Geometry of the plane kernel's plan: the run-time plan of the launch, or a compile-time constant for a shape
+// whose rows are whole aligned vectors (the launcher checks that the two agree before it picks the constant).
+struct PlaneGeoRuntime {
+  static constexpr bool kStatic = false;
+  static constexpr Plan2D plan() { return Plan2D{}; }
+};
+constexpr Plan2D static_plane_plan(int H, int W, int K, int L, int* tj1_out) {
+  Plan2D pl = make_plan2d_geometry(1, 1, H, W, K, L, false, 256, 1);
+  int tj1 = 4, sg_shift = 8;
+  choose_plane_shape(pl.h[1], pl.w[1], static_cast<size_t>(pl.plane_lds_floats) * 4, &tj1, &sg_shift);
+  while (sg_shift < 8 && static_cast<size_t>(pl.plane_lds_floats) * 4 * (256 >> sg_shift) > kLdsLimitBytes / 2) ++sg_shift;
+  finish_plane_plan(&pl, sg_shift);
+  if (tj1_out != nullptr) *tj1_out = tj1;
+  return pl;
+}
+template <int H, int W, int K, int L>
+struct PlaneGeoStatic {
+  static constexpr bool kStatic = true;
+  static constexpr Plan2D plan() { return static_plane_plan(H, W, K, L, nullptr); }
+  static constexpr int tj1() { int t = 4; static_plane_plan(H, W, K, L, &t); return t; }
+  static constexpr int mode() {
+    const Plan2D p = plan();
+    return (p.prefetch && p.fuse >= 2) ? 3 : p.prefetch ? 0 : p.vec_ok ? 1 : 2;
+  }
+};
+// Whether two plans describe the same LDS layout and work split (everything but batch and channels).
+inline bool same_plane_geometry(const Plan2D& a, const Plan2D& b) {
+  if (a.H != b.H || a.W != b.W || a.L != b.L || a.P != b.P || a.lds_floats != b.lds_floats || a.vec_ok != b.vec_ok ||
+      a.prefetch != b.prefetch || a.sg_shift != b.sg_shift || a.plane_lds_floats != b.plane_lds_floats ||
+      a.fuse != b.fuse || a.block != b.block)
+    return false;
+  for (int l = 0; l <= a.L; ++l)
+    if (a.h[l] != b.h[l] || a.w[l] != b.w[l] || a.aoff[l] != b.aoff[l] || a.astr[l] != b.astr[l] ||
+        a.apl[l] != b.apl[l] || a.zoff[l] != b.zoff[l] || a.zstr[l] != b.zstr[l])
+      return false;
+  return true;
+}
+
 // Planes per iteration of the weight-gradient kernel: as many (of one channel, consecutive
 // batch items, stacked vertically) as fit the LDS budget of two workgroups per CU, up to 16.
 // Small planes leave most of the 512 threads idle and pay the per-iteration barriers for
 // little work when taken one at a time (measured, bf16: 28x28 230 -> 197 us, 14x14 193 -> 160 us,
 // 7x7 148 -> 137 us); a 56x56 plane fills the budget by itself.
-inline int wgrad_planes_per_iter(int B, int H, int W, int K, int L) {
+constexpr int wgrad_planes_per_iter(int B, int H, int W, int K, int L) {
   int pb = B < 16 ? B : 16;
   if (pb < 1) pb = 1;
   while (pb > 1) {
-    const Plan2D t = make_plan2d(B, 1, H, W, K, L, true, 512, 4, nullptr, nullptr, nullptr, pb);
+    const Plan2D t = make_plan2d_geometry(B, 1, H, W, K, L, true, 512, pb);
     if (static_cast<size_t>(t.plane_lds_floats) * 4 <= 80 * 1024) break;
     --pb;
   }
@@ -129,7 +174,7 @@ inline int wgrad_planes_per_iter(int B, int H, int W, int K, int L) {
 }
 
 // Completes a plan for the weight-gradient kernel: threads per stacked plane, prefetch.
-inline void finish_wgrad_plan(Plan2D* pl, int K) {
+constexpr void finish_wgrad_plan(Plan2D* pl, int K) {
   // the final reduction reuses the LDS as [8 waves][sets * K * K + 1] floats, which is more
   // than the pyramids of a single tiny plane take
   const int red_floats = round_up(8 * (wgrad_sets(pl->L) * K * K + 1), 4);
@@ -144,6 +189,28 @@ inline void finish_wgrad_plan(Plan2D* pl, int K) {
     pl->prefetch = nps / gs >= pl->h[1];       // one 2x4 piece per thread covers the plane
     if (pl->prefetch && pl->pb == 1 && gs <= 16 && pl->L >= 2) pl->fuse = pl->L >= 3 ? 3 : 2;
   }
+}
+
+// Weight-gradient plan of a shape as a compile-time constant: PB planes per iteration, rows of whole aligned vectors.
+template <int H, int W, int K, int L, int PB>
+struct WgradGeoStatic {
+  static constexpr bool kStatic = true;
+  static constexpr Plan2D plan() {
+    Plan2D pl = make_plan2d_geometry(PB, 1, H, W, K, L, true, 512, PB);
+    finish_wgrad_plan(&pl, K);
+    return pl;
+  }
+};
+inline bool same_wgrad_geometry(const Plan2D& a, const Plan2D& b) {
+  if (a.H != b.H || a.W != b.W || a.L != b.L || a.P != b.P || a.lds_floats != b.lds_floats || a.vec_ok != b.vec_ok ||
+      a.prefetch != b.prefetch || a.pb != b.pb || a.slot_shift != b.slot_shift || a.fuse != b.fuse ||
+      a.plane_lds_floats != b.plane_lds_floats)
+    return false;
+  for (int l = 0; l <= a.L; ++l)
+    if (a.h[l] != b.h[l] || a.w[l] != b.w[l] || a.aoff[l] != b.aoff[l] || a.astr[l] != b.astr[l] ||
+        a.apl[l] != b.apl[l] || a.goff[l] != b.goff[l] || a.gstr[l] != b.gstr[l] || a.gpl[l] != b.gpl[l])
+      return false;
+  return true;
 }
 
 // ---- 1-D ------------------------------------------------------------------------------
