@@ -126,8 +126,9 @@ class _on_device:
         return False
 
 
-def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
-    """One forward launch sequence; returns (out, contiguous x)."""
+def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L, tabinfo=None):
+    """One forward launch sequence; returns (out, contiguous x).  `tabinfo`, a list, receives the
+    parameter table of the call for the backward pass to reuse."""
     lib = _lib.load()
     if not x.is_contiguous():
         x = x.contiguous()
@@ -138,6 +139,8 @@ def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
         out, _ = _forward_impl(x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L)
         return out.to(torch.float16), x
     pd, tab, _keep = _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    if tabinfo is not None:
+        tabinfo.append((pd, tab, _keep))
     shape = tuple(x.shape)
     with _on_device(x.device):
         out = torch.empty_like(x)
@@ -152,7 +155,7 @@ def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L):
     return out, x
 
 
-def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L, need_x, need_params):
+def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L, need_x, need_params, tabinfo=None):
     """grad_x (or None) and the parameter gradients in the order base_w, base_b (or None),
     base_s, wt_ws[0..L-1], wt_ss[0..L-1] (all None when not needed), in the parameters' dtypes."""
     lib = _lib.load()
@@ -165,7 +168,8 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
         g = g.to(x.dtype)
     if not g.is_contiguous():
         g = g.contiguous()
-    pd, tab, _keep = _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
+    # (the forward pass's table of the same, unmodified tensors, when it left one)
+    pd, tab, _keep = tabinfo if tabinfo is not None else _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
     has_bias = base_b is not None
     shape = tuple(x.shape)
     grad_x = None
@@ -180,13 +184,17 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
         if need_x:
             grad_x = torch.empty_like(x)
         if need_params:
-            # one flat fp32 buffer for every gradient: a single allocation and, for bf16
-            # parameters, a single cast afterwards
             plist = [base_w, base_s] + ([base_b] if has_bias else []) + list(wt_ws) + list(wt_ss)
-            sizes = [t.numel() for t in plist]
-            flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
-            views = flat.split(sizes)
             nb = 3 if has_bias else 2
+            same_f32 = all(t.dtype == torch.float32 for t in plist)
+            if same_f32:
+                # fp32 parameters: every gradient is written in place, in its parameter's shape
+                views = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in plist]
+            else:
+                # other parameter dtypes: one flat fp32 buffer, so that one cast serves every gradient
+                sizes = [t.numel() for t in plist]
+                flat = torch.empty(sum(sizes), dtype=torch.float32, device=x.device)
+                views = flat.split(sizes)
             gtab = _table(_lib.ParamGrads, views[0], views[2] if has_bias else None, views[1],
                           views[nb:nb + L], views[nb + L:])
         if need_x and need_params:        # the whole backward pass in one library call
@@ -208,15 +216,16 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
             if rc:
                 _lib.check(rc, "wtconv backward_params")
         if need_params:
-            tensors = [base_w, base_s] + ([base_b] if base_b is not None else []) + list(wt_ws) + list(wt_ss)
-            out_dt = base_w.dtype
-            if all(t.dtype == out_dt for t in tensors):
-                cast = flat.to(out_dt).split(sizes) if out_dt != torch.float32 else views
-                outg = [v.view(t.shape) for v, t in zip(cast, tensors)]
+            if same_f32:
+                outg = views
             else:
-                outg = [v.to(t.dtype).view(t.shape) for v, t in zip(views, tensors)]
+                out_dt = base_w.dtype
+                if all(t.dtype == out_dt for t in plist):
+                    outg = [v.view(t.shape) for v, t in zip(flat.to(out_dt).split(sizes), plist)]
+                else:
+                    outg = [v.to(t.dtype).view(t.shape) for v, t in zip(views, plist)]
             grads[0], grads[2] = outg[0], outg[1]
-            if base_b is not None:
+            if has_bias:
                 grads[1] = outg[2]
             for i in range(L):
                 grads[3 + i] = outg[nb + i]
@@ -230,24 +239,26 @@ class _WTConvFn(torch.autograd.Function):
 
     # Under torch.autocast the inputs are taken as they come (fp32 or bf16 activations, fp32 or
     # bf16 parameters, any mix): the kernels accumulate in fp32 either way, so there is nothing
-    # to down-cast; the decorators only make backward run with autocast off, as forward did.
+    # to down-cast, and neither pass runs a torch operator that autocast would touch (hence no
+    # custom_fwd / custom_bwd wrappers: entering an autocast context costs more host time than the
+    # rest of the backward prelude).
     @staticmethod
-    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, x, base_w, base_b, base_s, dims, K, L, *wt):
-        out, x = _forward_impl(x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L)
+        info = []
+        out, x = _forward_impl(x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L, info)
         ctx.dims, ctx.K, ctx.L = dims, K, L
+        ctx.tabinfo = info[0] if info and x.dtype != torch.float16 else None
         ctx.save_for_backward(x, base_w, base_b, base_s, *wt)
         return out
 
     @staticmethod
     @torch.autograd.function.once_differentiable      # double backward raises instead of being silently wrong
-    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_out):
         x, base_w, base_b, base_s, *wt = ctx.saved_tensors
         dims, K, L = ctx.dims, ctx.K, ctx.L
         need_params = any(ctx.needs_input_grad[i] for i in (1, 2, 3)) or any(ctx.needs_input_grad[7:])
         grad_x, grads = _backward_impl(grad_out, x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L,
-                                       ctx.needs_input_grad[0], need_params)
+                                       ctx.needs_input_grad[0], need_params, ctx.tabinfo)
         return (grad_x, grads[0], grads[1], grads[2], None, None, None, *grads[3:])
 
 
