@@ -134,6 +134,10 @@ def test_emulated_2d_mfma_fp32_split(B, C, H, W, K, L, bias):
     (3, 2, 28, 28, 5, 3, True, 0),
     (2, 2, 14, 14, 5, 2, False, 0),
     (1, 1, 56, 56, 5, 3, True, 0),
+    (2, 2, 7, 7, 5, 2, False, 0),      # gradients: fewer row tiles than lane groups (idle groups read zeros)
+    (3, 1, 9, 13, 3, 3, True, 0),      # gradients: K = 3 in the 5 x 5 frame, odd sizes, level 3 through LDS
+    (1, 1, 64, 64, 5, 3, True, 0),     # gradients: a single plane beyond the LDS of two workgroups (eight waves)
+    (2, 1, 33, 20, 1, 2, True, 1),     # gradients: K = 1, two column tiles at level 0
 ])
 def test_emulated_2d_mfma_bf16(B, C, H, W, K, L, bias, pdtype):
     x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias, dtype=1, pdtype=pdtype)
