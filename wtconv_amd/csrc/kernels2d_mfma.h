@@ -281,13 +281,31 @@ __device__ __forceinline__ void fold_entry(const ParamTable& p, int pdtype, int 
 #pragma unroll 1
       for (int i = 0; i <= l; ++i) scale *= 0.25f;
     }
-    if (ih >= 0 && ih < K) {
+    // the (up to five) taps of the entry's kernel row, fetched together whether or not the entry uses them: loads
+    // behind per-tap conditions would complete one after the other, and a channel switch waits for this fold
+    const bool row_ok = ih >= 0 && ih < K;
+    const int frow = row_ok ? (flip ? K - 1 - ih : ih) : 0;
+    const int rowi = ch * KK + frow * K;
+    float wr[5];
+    if (pdtype == WTCONV_F32) {
+      const float* w = static_cast<const float*>(wp) + rowi;
+#pragma unroll
+      for (int i = 0; i < 5; ++i) wr[i] = w[i < K ? i : K - 1];
+    } else {
+      const bf16_t* w = static_cast<const bf16_t*>(wp) + rowi;
+#pragma unroll
+      for (int i = 0; i < 5; ++i) wr[i] = bf16_to_f32(w[i < K ? i : K - 1]);
+    }
+    if (row_ok) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int iw = j - cs - o;
         if (iw >= 0 && iw < K && j - cs < 5 && j - cs >= 0) {
-          const int t = ih * K + iw;
-          v[j] = load_param(wp, pdtype, ch * KK + (flip ? KK - 1 - t : t)) * scale;
+          const int fi = flip ? K - 1 - iw : iw;
+          float t = wr[0];
+#pragma unroll
+          for (int i = 1; i < 5; ++i) t = fi == i ? wr[i] : t;
+          v[j] = t * scale;
         }
       }
     }
