@@ -123,6 +123,28 @@ def test_stage_shapes_bf16_small_batch(hip_device, C, H, L, bf16_params):
     U.compare_all(got, want, U.assert_bf16)
 
 
+@pytest.mark.parametrize("B,H,L", [(2, 56, 3), (8, 28, 3), (24, 14, 2), (58, 7, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_stage_planes_at_the_batch_of_their_compile_time_plans(hip_device, B, H, L, dtype):
+    """The four stage plane sizes with enough batch items that the kernels take the planes-per-unit of their
+    compile-time plans (1, 4, 11, 29 forward; 1, 3, 12, 24 and 1, 3, 12, 16 for the gradients), few channels:
+    every output and gradient against the oracle."""
+    W2, _ = _mods()
+    C = 4
+    ref, x, g = U.seeded_case("2d", C, 5, L, (B, C, H, H), seed=3)
+    U.randomize_scales(ref)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, L)
+    if dtype == torch.bfloat16:
+        x, g = x.to(dtype).float(), g.to(dtype).float()
+        got = U.hip_run(mod, x, g, hip_device, dtype=dtype)
+        want = U.oracle_run(ref, x, g, torch.float32)
+        U.compare_all(got, want, U.assert_bf16)
+    else:
+        got = U.hip_run(mod, x, g, hip_device)
+        want = U.oracle_run(ref, x, g, torch.float64)
+        U.compare_all(got, want, U.assert_fp32)
+
+
 def test_large_plane_bf16(hip_device):
     """mmseg-sized plane (128x128, five levels) in bf16: the level-by-level kernels keep the
     pyramid in fp32, so the bf16 bar applies to the rounding at the HBM boundary only."""

@@ -698,7 +698,7 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
         mma_tile<NS>(at, ab, bt, bb, acc);
       }
     };
-    const bool early = ntile1 <= 4 && L >= 2 && wave < 3;   // this wave's single level-1 tile starts before the barrier
+    const bool early = ntile1 <= 4 && L >= 2;   // every wave's single level-1 tile starts before the barrier
     TileLane tl1 = {};
     Acc acc1[4];
 #pragma unroll
@@ -791,11 +791,13 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
           lds_st<float4>(lds, zoff1 + (imul(tl.p, zpl1) + imul(4 * tl.bi + q, zpitch1) + 4 * tl.tc) * 4, a);
         }
       }
-      if (early && wave < ntile1) {
-        tl1 = tile_lane(lds, wave, n, q, tcs1, nrow1, nbc1, rtoff1, aoff1, pitchB1);
+    }
+    // the detail sub-bands of this wave's level-1 tile: they need nothing of this stage (the coarse-chain wave
+    // runs them after its chain, which is shorter than the base-conv share of the others)
+    if (early && wave < ntile1) {
+      tl1 = tile_lane(lds, wave, n, q, tcs1, nrow1, nbc1, rtoff1, aoff1, pitchB1);
 #pragma unroll
-        for (int s = 1; s < 4; ++s) conv1(tl1, s, acc1[s]);
-      }
+      for (int s = 1; s < 4; ++s) conv1(tl1, s, acc1[s]);
     }
     WT_LDS_BARRIER();
 
