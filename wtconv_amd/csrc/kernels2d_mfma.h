@@ -327,11 +327,19 @@ __device__ __forceinline__ void fold_entry(const ParamTable& p, int pdtype, int 
 template <typename T> struct PixRow;
 template <> struct PixRow<float> { float4 v; };
 template <> struct PixRow<bf16_t> { uint2 v; };
-// bf16 pixels fetched one by one (rows that are not whole aligned vectors): each in a register of its own, as
-// it comes from memory -- nothing is computed on them before use, so all the loads of a block stay in flight.
-struct PixRowU { uint32_t e[4]; };
-template <typename T, bool VEC> struct PixSel { using type = PixRow<T>; };
-template <> struct PixSel<bf16_t, false> { using type = PixRowU; };
+// Rows of bf16 planes that are not whole aligned vectors still move as one 8-byte access per row of a block: global
+// memory takes unaligned accesses (the compiler itself emits one dwordx2 for an 8-byte copy from a 2-byte aligned
+// address).  Columns past the row end come along and are cleared before use; nothing is computed on the loaded
+// words before the commit, so all the loads of a block stay in flight.
+__device__ __forceinline__ void pix_load4u(uint2& v, const bf16_t* p) { __builtin_memcpy(&v, p, 8); }
+__device__ __forceinline__ void pix_store4u(bf16_t* p, const uint2& v) { __builtin_memcpy(p, &v, 8); }
+// words that keep the valid columns of a block row: bits 4..7 of `cmask` say which of its four columns exist
+__device__ __forceinline__ uint2 pix_col_mask(unsigned cmask) {
+  uint2 m;
+  m.x = ((cmask & 16u) ? 0x0000ffffu : 0u) | ((cmask & 32u) ? 0xffff0000u : 0u);
+  m.y = ((cmask & 64u) ? 0x0000ffffu : 0u) | ((cmask & 128u) ? 0xffff0000u : 0u);
+  return m;
+}
 
 __device__ __forceinline__ void pix_zero(PixRow<float>& r) { r.v.x = r.v.y = r.v.z = r.v.w = 0.f; }
 __device__ __forceinline__ void pix_zero(PixRow<bf16_t>& r) { r.v.x = r.v.y = 0u; }
@@ -344,19 +352,8 @@ __device__ __forceinline__ void pix_set(PixRow<bf16_t>& r, int i, bf16_t v) {
   const uint32_t u = static_cast<uint32_t>(v) << ((i & 1) * 16);
   if (i < 2) r.v.x |= u; else r.v.y |= u;
 }
-__device__ __forceinline__ void pix_zero(PixRowU& r) { r.e[0] = r.e[1] = r.e[2] = r.e[3] = 0u; }
-__device__ __forceinline__ void pix_load4(PixRowU&, const bf16_t*) {}      // (never taken: vector rows use PixRow)
-__device__ __forceinline__ void pix_set(PixRowU& r, int i, bf16_t v) { r.e[i] = v; }
-__device__ __forceinline__ void pix_get(const PixRowU& r, float (&f)[4]) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r.e[i] << 16);
-}
 // the four bf16 of a row as two packed words
 __device__ __forceinline__ uint2 pix_words(const PixRow<bf16_t>& r) { return r.v; }
-__device__ __forceinline__ uint2 pix_words(const PixRowU& r) {
-  uint2 w; w.x = r.e[0] | (r.e[1] << 16); w.y = r.e[2] | (r.e[3] << 16);
-  return w;
-}
 __device__ __forceinline__ uint2 pix_words(const PixRow<float>&) { uint2 w; w.x = w.y = 0u; return w; }   // (never taken)
 __device__ __forceinline__ void pix_get(const PixRow<float>& r, float (&f)[4]) {
   f[0] = r.v.x; f[1] = r.v.y; f[2] = r.v.z; f[3] = r.v.w;
@@ -522,11 +519,13 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   const int u_begin = static_cast<int>(static_cast<long long>(blockIdx.x) * pl.nunits / G);
   const int u_end = static_cast<int>(static_cast<long long>(blockIdx.x + 1) * pl.nunits / G);
 
-  typename PixSel<T, VEC>::type pf[NBL][4];
+  PixRow<T> pf[NBL][4];
+  const size_t total_elems = static_cast<size_t>(B) * C * HW;
   auto fetch = [&](int u) {
     const int c = u / upc;
     const int b0 = (u - c * upc) * pb;
-    const T* base = x + (static_cast<size_t>(b0) * C + c) * HW;
+    const size_t base_off = (static_cast<size_t>(b0) * C + c) * HW;
+    const T* base = x + base_off;
 #pragma unroll
     for (int i = 0; i < NBL; ++i) {
       const bool plane_ok = (c_mask[i] & 0x100u) && b0 + c_p[i] < B;
@@ -537,6 +536,16 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
           const T* src = base + c_goff[i] + r * W;
           if constexpr (VEC) {
             if (c_mask[i] & 16u) pix_load4(pf[i][r], src);
+          } else if constexpr (sizeof(T) == 2) {
+            // one unaligned 8-byte load per row (columns past the row end are cleared at the commit); only a row
+            // whose four elements would reach past the end of the tensor goes element by element
+            if (base_off + c_goff[i] + r * W + 4 <= total_elems) {
+              pix_load4u(pf[i][r].v, src);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (c_mask[i] >> (4 + e) & 1u) pix_set(pf[i][r], e, src[e]);
+            }
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -592,6 +601,11 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
     for (int i = 0; i < NBL; ++i) {
       if (!(c_mask[i] & 0x100u)) continue;
       float v[4][4];
+      if constexpr (!VEC && sizeof(T) == 2) {      // clear the columns that came along from past the row end
+        const uint2 m = pix_col_mask(c_mask[i]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { pf[i][r].v.x &= m.x; pf[i][r].v.y &= m.y; }
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) pix_get(pf[i][r], v[r]);
 #pragma unroll
@@ -857,6 +871,16 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
                 } else {
                   uint2 o2; o2.x = pack_bf16x2(r0, r1); o2.y = pack_bf16x2(r2, r3);
                   *reinterpret_cast<uint2*>(dst) = o2;
+                }
+              } else if constexpr (sizeof(T) == 2) {
+                if (x0 + 3 < W) {      // four columns inside the row: one (unaligned) 8-byte store
+                  uint2 o2; o2.x = pack_bf16x2(r0, r1); o2.y = pack_bf16x2(r2, r3);
+                  pix_store4u(dst, o2);
+                } else {
+                  const float r[4] = {r0, r1, r2, r3};
+#pragma unroll
+                  for (int e = 0; e < 4; ++e)
+                    if (x0 + e < W) dst[e] = from_f32<T>(r[e]);
                 }
               } else {
                 const float r[4] = {r0, r1, r2, r3};

@@ -231,9 +231,11 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
   const int xsub2 = pl.xsub[L >= 2 ? 2 : 0], gsub2 = pl.gsub[L >= 2 ? 2 : 0];
   const int llx2 = pl.llxoff[L >= 3 ? 2 : 0], llg2 = pl.llgoff[L >= 3 ? 2 : 0];
 
-  using Pix = typename PixSel<bf16_t, VEC>::type;
+  using Pix = PixRow<bf16_t>;
   Pix px[4], pg[kSplitCommit ? 1 : 4];
   const bf16_t* src0 = (kSplitCommit && half) ? g : x;
+  const size_t total_elems = static_cast<size_t>(B) * C * HW;
+  const uint2 colmask = pix_col_mask(cmask);
   auto fetch = [&](int b0) {
     const size_t base = (static_cast<size_t>(b0) * C + c) * HW;
     const bool plane_ok = act && b0 + cp < b_end;
@@ -249,7 +251,12 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
             pix_load4(px[r], sx);
             if constexpr (!kSplitCommit) pix_load4(pg[r], sg);
           }
-        } else {
+        } else if (base + c_goff + r * W + 4 <= total_elems) {
+          // rows that are not whole aligned vectors: still one (unaligned) 8-byte load per row; the columns that
+          // come along from past the row end are cleared at the commit
+          pix_load4u(px[r].v, sx);
+          if constexpr (!kSplitCommit) pix_load4u(pg[r].v, sg);
+        } else {      // the four elements would reach past the end of the tensor: element by element
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (cmask >> (4 + e) & 1u) {
@@ -274,11 +281,16 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
                     int sub2, int llo, float& llsum, auto n1) {
     constexpr int N1 = decltype(n1)::value;
     float v[4][4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) pix_get(pr[r], v[r]);
+    Pix row[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const uint2 w = pix_words(pr[r]);
+      row[r] = pr[r];
+      if constexpr (!VEC) { row[r].v.x &= colmask.x; row[r].v.y &= colmask.y; }
+      pix_get(row[r], v[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const uint2 w = pix_words(row[r]);
       if (pair64) {
         lds_st<uint2>(lds, o0 + r * pitch0 * 2, w);
       } else {
@@ -330,7 +342,7 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
 #pragma unroll
     for (int l = 0; l < L; ++l) dl[l][k].v[0] = dl[l][k].v[1] = dl[l][k].v[2] = dl[l][k].v[3] = 0.f;
   }
-  float gsum = 0.f, unused = 0.f;
+  float gsum = 0.f, no_sum = 0.f;      // (the LL sum of x is not needed)
 
   // one level of both pyramids from the raw LL of the level above (fp32 in LDS)
   auto analyse = [&](auto lc) {
@@ -417,7 +429,7 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     if (act) {
       using std::integral_constant;
       if (!kSplitCommit || half == 0)
-        commit(px, x_l0, pl.xpitch[0], true, x_l1, pl.xpitch[1], pl.xsub[1], x_l2, xsub2, llx2 + ll_i, unused,
+        commit(px, x_l0, pl.xpitch[0], true, x_l1, pl.xpitch[1], pl.xsub[1], x_l2, xsub2, llx2 + ll_i, no_sum,
                integral_constant<int, 2>{});
       if constexpr (kSplitCommit) {
         if (half == 1)
