@@ -817,8 +817,8 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
 
     // ---- stage 2: level 1 (conv, inverse Haar), plus the base conv from Z_1, to HBM
     {
-      WT_WAIT_VMEM();       // the prefetch has landed; the stores below then drain behind the next unit's work
       T* obase = out + (static_cast<size_t>(b0) * C + c) * HW;
+      bool first_store = true;
 #pragma unroll 1
       for (int t = wave; t < ntile1; t += 4) {
         if (!early) {
@@ -850,6 +850,12 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
         }
         float top[8], bot[8];
         synth_rows(acc1, top, bot);
+        if (first_store) {
+          // the prefetch of the next unit has had this tile's convolutions to land; waiting for it here, ahead of
+          // the first store, lets the stores drain behind the next unit's work instead of being waited for at its commit
+          WT_WAIT_VMEM();
+          first_store = false;
+        }
         if (store_ok) {
           T* dbase = obase + static_cast<size_t>(tl1.p) * C * HW + imul(y, W) + xx;
 #pragma unroll
