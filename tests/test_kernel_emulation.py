@@ -147,6 +147,26 @@ def test_emulated_2d_mfma_bf16(B, C, H, W, K, L, bias, pdtype):
     _compare(got, want, rtol=2e-2, atol_scale=2e-2)
 
 
+def _random_mfma_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        H, W = rnd.randint(1, 26), rnd.randint(1, 26)
+        L = rnd.randint(1, 4)
+        cases.append((rnd.randint(1, 5), rnd.randint(1, 2), H, W, rnd.choice([1, 3, 5]), L, rnd.random() < 0.7))
+    return cases
+
+
+@pytest.mark.parametrize("B,C,H,W,K,L,bias", _random_mfma_cases(14, 20241))
+def test_emulated_2d_mfma_bf16_random_shapes(B, C, H, W, K, L, bias):
+    """Seeded random small shapes through the matrix-core kernels (forward, input gradient, parameter gradients)
+    under the address sanitizer: every narrow-level variant of the gradient tiles, idle lane groups, ragged units."""
+    x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias, dtype=1, pdtype=0)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, K, dtype=1, pdtype=0, mfma=1)
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-2, atol_scale=2e-2)
+
+
 def test_emulated_2d_bf16_vector_alu_kernels():
     """bf16 tensors on the vector-ALU kernels (what K = 7 or planes wider than 64 take)."""
     x, g, bw, bb, bs, ws, ss = _case2d(1, 2, 8, 12, 5, 2, True, dtype=1, pdtype=1)
