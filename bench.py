@@ -56,7 +56,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--dtype", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--dtype", choices=["fp32", "bf16", "fp16"], default="fp32")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="stage1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary dtype and per-kernel timing")
@@ -155,13 +155,13 @@ def bench_layer(torch, dev, dtype_name, workload, steps, warmup, per_kernel=True
     from wtconv_amd import _lib
     from wtconv_amd import functional as Fn
     C, H, W, K, L, B = WORKLOADS[workload]
-    dtype = torch.float32 if dtype_name == "fp32" else torch.bfloat16
+    dtype = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dtype_name]
     esz = 4 if dtype_name == "fp32" else 2
     P = B * C * H * W
     torch.manual_seed(0)
     mod = wtconv.WTConv2d(C, C, K, wt_levels=L).to(dev)
     if dtype_name == "bf16":
-        mod = mod.to(torch.bfloat16)
+        mod = mod.to(torch.bfloat16)      # (fp16 activations keep fp32 parameters, as under torch.autocast)
     set_bytes = 3 * P * esz
     nsets = max(3, int(600e6 // set_bytes) + 1)
     sets = make_sets(torch, dev, dtype, C, H, W, B, nsets)
@@ -405,7 +405,7 @@ def main():
     C, H, W, K, L, B = WORKLOADS[args.workload]
 
     if args.probe_copy:
-        dt = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+        dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[args.dtype]
         src = torch.randn(B, C, H, W, device=dev).to(dt)
         dst = torch.empty_like(src)
         for _ in range(args.warmup + args.steps):
@@ -431,7 +431,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.dtype == "fp32" else "bf16",
+        "dtype": {"fp32": "f32", "bf16": "bf16", "fp16": "f16 in HBM, f32 arithmetic"}[args.dtype],
         "data": "synthetic",
         "config": {"workload": f"WTConv2d({C},{C},kernel_size={K},wt_levels={L}) fwd+bwd on x[{B},{C},{H},{W}] "
                                f"({args.workload}), all parameter grads, seeded default init"},
@@ -457,6 +457,11 @@ def main():
         line["other_dtype"] = {k: o[k] for k in keys if k in o}
         if "kernels" in o:
             line["other_dtype"]["roofline"] = roofline_of(o["kernels"], args.workload, other, K, L, B * C * H * W)
+        if args.workload == "stage1" and args.dtype != "fp16":
+            # fp16 tensors take the vector kernels: fp16 in HBM, fp32 arithmetic
+            o = bench_layer(torch, dev, "fp16", args.workload, max(10, args.steps // 2), max(3, args.warmup // 2),
+                            per_kernel=False)
+            line["fp16"] = {k: o[k] for k in keys if k in o}
         if args.workload == "stage1":
             sweep = {}
             for wl in ("stage2", "stage3", "stage4"):

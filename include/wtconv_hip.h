@@ -7,7 +7,9 @@
  *     caller; the library never allocates, frees or synchronises, and launches on the
  *     HIP stream handed in (`stream`, a hipStream_t passed as void*; NULL = default);
  *   - activations are contiguous NCHW (2-D) / NCL (1-D) in `dtype`; parameters are
- *     contiguous in `param_dtype`; parameter gradients are always written as float;
+ *     contiguous in `param_dtype`; parameter gradients are always written as float.
+ *     The three element types are those the reference's fused twin dispatches
+ *     (fast_wtconv/cuda_haar/haar_common.cuh:55-77): float, bfloat16 and IEEE half;
  *   - return value 0 on success, a negative WTCONV_E_* code otherwise, with a message
  *     retrievable from wtconv_last_error() on the calling thread;
  *   - `workspace` must hold at least wtconv*_workspace_bytes(...) bytes, 256-byte aligned.
@@ -26,9 +28,9 @@ extern "C" {
 #endif
 
 #define WTCONV_MAX_LEVELS 5
-#define WTCONV_ABI_VERSION 3
+#define WTCONV_ABI_VERSION 4
 
-enum { WTCONV_F32 = 0, WTCONV_BF16 = 1 };
+enum { WTCONV_F32 = 0, WTCONV_BF16 = 1, WTCONV_F16 = 2 };
 
 enum {
   WTCONV_OK = 0,

@@ -5,7 +5,10 @@
 // in.bin : int32 header {dims, B, C, H, W, K, L, dtype, pdtype, has_bias}, then float32
 //          arrays x, g, base_w, base_b (if has_bias), base_s, then per level w_l, s_l.
 // out.bin: float32 arrays out, dx, dbase_w, dbase_b (if has_bias), dbase_s, per level dw_l, ds_l.
-// With dtype/pdtype = 1 the driver rounds the arrays to bfloat16 storage first.
+// dims == 0: in.bin holds B floats after the header; out.bin receives each after a round trip through the kernels'
+//          float -> half -> float conversions.
+// With dtype/pdtype = 1 the driver rounds the arrays to bfloat16 storage first, with 2 to IEEE half.
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -13,6 +16,7 @@
 #include <vector>
 
 #include "../../include/wtconv_hip.h"
+#include "../../wtconv_amd/csrc/common.h"      // only for the half conversions of the dims == 0 mode
 
 static uint16_t to_bf16(float f) {
   uint32_t u; std::memcpy(&u, &f, 4);
@@ -21,13 +25,34 @@ static uint16_t to_bf16(float f) {
 }
 static float from_bf16(uint16_t v) { uint32_t u = static_cast<uint32_t>(v) << 16; float f; std::memcpy(&f, &u, 4); return f; }
 
+// IEEE half by way of the value: nearest multiple of the half's spacing at that magnitude (ties to even)
+static uint16_t to_f16(float f) {
+  const uint16_t sign = std::signbit(f) ? 0x8000u : 0u;
+  const double a = std::fabs(static_cast<double>(f));
+  if (std::isnan(f)) return sign | 0x7e00u;
+  if (a >= 65520.0) return sign | 0x7c00u;
+  int e = a > 0 ? std::ilogb(a) : -14;
+  if (e < -14) e = -14;
+  const double q = std::nearbyint(std::ldexp(a, 10 - e));      // in units of 2^(e-10); default rounding is to even
+  uint32_t m = static_cast<uint32_t>(q);
+  uint32_t bits = (e == -14 && m < 1024u) ? m : ((static_cast<uint32_t>(e + 15) << 10) + (m - 1024u));
+  return static_cast<uint16_t>(sign | bits);
+}
+static float from_f16(uint16_t h) {
+  const int ex = (h >> 10) & 31, man = h & 1023;
+  double v = ex == 31 ? (man ? NAN : INFINITY) : ex == 0 ? std::ldexp(man, -24) : std::ldexp(1024 + man, ex - 25);
+  return static_cast<float>((h & 0x8000u) ? -v : v);
+}
+
 struct Buf {
   std::vector<float> f;       // float view (input as read / output to write)
-  std::vector<uint16_t> h;    // bf16 storage when dtype == 1
+  std::vector<uint16_t> h;    // bf16 storage when dtype == 1, half storage when dtype == 2
   int dtype = 0;
   void* ptr() { return dtype ? static_cast<void*>(h.data()) : static_cast<void*>(f.data()); }
-  void pack() { if (dtype) { h.resize(f.size()); for (size_t i = 0; i < f.size(); ++i) h[i] = to_bf16(f[i]); } }
-  void unpack() { if (dtype) for (size_t i = 0; i < f.size(); ++i) f[i] = from_bf16(h[i]); }
+  void pack() {
+    if (dtype) { h.resize(f.size()); for (size_t i = 0; i < f.size(); ++i) h[i] = dtype == 2 ? to_f16(f[i]) : to_bf16(f[i]); }
+  }
+  void unpack() { if (dtype) for (size_t i = 0; i < f.size(); ++i) f[i] = dtype == 2 ? from_f16(h[i]) : from_bf16(h[i]); }
 };
 
 static Buf read_buf(FILE* fp, size_t n, int dtype) {
@@ -46,6 +71,17 @@ int main(int argc, char** argv) {
   if (fread(hd, 4, 10, fp) != 10) return 2;
   const int dims = hd[0], B = hd[1], C = hd[2], H = hd[3], W = hd[4], K = hd[5], L = hd[6];
   const int dtype = hd[7], pdtype = hd[8], has_bias = hd[9];
+  if (dims == 0) {
+    std::vector<float> v(B);
+    if (B && fread(v.data(), 4, v.size(), fp) != v.size()) return 2;
+    fclose(fp);
+    for (float& f : v) f = wt::f16_bits_to_f32(wt::f32_to_f16_bits(f));
+    FILE* fo = fopen(argv[2], "wb");
+    if (!fo) { perror("open"); return 2; }
+    fwrite(v.data(), 4, v.size(), fo);
+    fclose(fo);
+    return 0;
+  }
   const int S = dims == 2 ? 4 : 2;
   const size_t KK = dims == 2 ? static_cast<size_t>(K) * K : K;
   const size_t P = static_cast<size_t>(B) * C * H * W;   // 1-D: H == 1, W == N

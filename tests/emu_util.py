@@ -32,6 +32,23 @@ def build(force=False):
     return EXE
 
 
+def half_roundtrip(values):
+    """float32 array -> the kernels' emulated float -> half -> float conversions of each element."""
+    exe = build()
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    hdr = np.array([0, v.size, 0, 0, 0, 0, 0, 0, 0, 0], dtype=np.int32)
+    with tempfile.TemporaryDirectory() as td:
+        fin, fout = os.path.join(td, "in.bin"), os.path.join(td, "out.bin")
+        with open(fin, "wb") as f:
+            f.write(hdr.tobytes() + v.tobytes())
+        env = dict(os.environ)
+        env["ASAN_OPTIONS"] = "detect_leaks=0"
+        r = subprocess.run([exe, fin, fout], capture_output=True, text=True, timeout=120, env=env)
+        if r.returncode != 0:
+            raise RuntimeError(f"emu_driver failed ({r.returncode}):\n{r.stderr[-4000:]}")
+        return np.fromfile(fout, dtype=np.float32)
+
+
 def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600, lds_limit=None,
         mfma=None):
     """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays.

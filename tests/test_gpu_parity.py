@@ -124,7 +124,7 @@ def test_stage_shapes_bf16_small_batch(hip_device, C, H, L, bf16_params):
 
 
 @pytest.mark.parametrize("B,H,L", [(2, 56, 3), (8, 28, 3), (24, 14, 2), (58, 7, 2)])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_stage_planes_at_the_batch_of_their_compile_time_plans(hip_device, B, H, L, dtype):
     """The four stage plane sizes with enough batch items that the kernels take the planes-per-unit of their
     compile-time plans (1, 4, 11, 29 forward; 1, 3, 12, 24 and 1, 3, 12, 16 for the gradients), few channels:
@@ -139,6 +139,18 @@ def test_stage_planes_at_the_batch_of_their_compile_time_plans(hip_device, B, H,
         got = U.hip_run(mod, x, g, hip_device, dtype=dtype)
         want = U.oracle_run(ref, x, g, torch.float32)
         U.compare_all(got, want, U.assert_bf16)
+    elif dtype == torch.float16:          # fp16 in HBM, fp32 arithmetic: results to fp16 rounding, parameter gradients to the fp32 bar
+        x, g = x.to(dtype).float(), g.to(dtype).float()
+        got = U.hip_run(mod, x, g, hip_device, dtype=dtype)
+        want = U.oracle_run(ref, x, g, torch.float64)
+
+        def check(a, b, name):
+            if name in ("out", "grad_x"):
+                rms = b.double().pow(2).mean().sqrt().item()
+                torch.testing.assert_close(a.double(), b.double(), rtol=2e-3, atol=2e-3 * rms, msg=lambda m: f"{name}: {m}")
+            else:
+                U.assert_fp32(a, b, name)
+        U.compare_all(got, want, check)
     else:
         got = U.hip_run(mod, x, g, hip_device)
         want = U.oracle_run(ref, x, g, torch.float64)
@@ -221,17 +233,26 @@ def test_under_autocast_and_channels_last(hip_device):
     U.assert_bf16(half_in.float().cpu(), plain.cpu(), "bf16 activations under autocast")
 
 
-@pytest.mark.parametrize("kind,shape,L", [("2d", (2, 8, 20, 22), 2), ("1d", (2, 4, 300), 3)])
-def test_fp16_activations(hip_device, kind, shape, L):
-    """float16 activations (the default AMP dtype of the reference's trainer, train.py:180,438):
-    oracle = fp32 maths on the fp16-rounded inputs; bar = rounding of the result to fp16
-    (rtol 2e-3, atol 2e-3 of the oracle's RMS); parameter gradients, which stay fp32, to the fp32 bar."""
+@pytest.mark.parametrize("kind,shape,K,L", [
+    ("2d", (2, 8, 20, 22), 5, 2),        # element-wise rows
+    ("2d", (3, 4, 56, 56), 5, 3),        # rows of whole vectors (the stage-1 plane)
+    ("2d", (2, 3, 17, 31), 7, 3),        # odd sizes, K = 7
+    ("2d", (1, 2, 230, 250), 3, 2),      # beyond LDS: the level-by-level kernels
+    ("1d", (2, 4, 300), 5, 3),           # short rows: tiled kernels
+    ("1d", (2, 3, 4096), 5, 4),          # row-resident kernels, vector rows
+    ("1d", (1, 2, 1001), 3, 5),          # row-resident, scalar rows
+])
+def test_fp16_activations(hip_device, kind, shape, K, L):
+    """float16 activations (the default AMP dtype of the reference's trainer, train.py:180,438; the reference's fused
+    twin dispatches the type too, haar_common.cuh:55-77): the kernels read and write fp16 and compute in fp32.
+    Oracle = float64 maths on the fp16-rounded inputs; bar = rounding of the result to fp16 (rtol 2e-3, atol 2e-3
+    of the oracle's RMS); parameter gradients, which stay fp32, to the fp32 bar."""
     W2, W1 = _mods()
-    ref, x, g = U.seeded_case(kind, shape[1], 5, L, shape)
+    ref, x, g = U.seeded_case(kind, shape[1], K, L, shape)
     U.randomize_scales(ref)
     rh = lambda t: t.to(torch.float16).float()
     x, g = rh(x), rh(g)
-    mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, 5, L)
+    mod = U.copy_to_hip_module(ref, W2 if kind == "2d" else W1, kind, K, L)
     out, dx, grads = U.hip_run(mod, x, g, hip_device, dtype=torch.float16)
     wo, wdx, wg = U.oracle_run(ref, x, g, torch.float64)
 
@@ -242,6 +263,29 @@ def test_fp16_activations(hip_device, kind, shape, L):
     close16(dx, wdx, "grad_x")
     for n, v in grads.items():
         U.assert_fp32(v, wg[n], n)
+
+
+def test_fp16_module_half_parameters(hip_device):
+    """A module converted with .half(): fp16 parameters are read as they are and their gradients come back as fp16."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 6, 5, 2, (2, 6, 24, 28))
+    U.randomize_scales(ref)
+    rh = lambda t: t.to(torch.float16).float()
+    for p in ref.parameters():
+        p.data = rh(p.data)
+    x, g = rh(x), rh(g)
+    mod = U.copy_to_hip_module(ref, W2, "2d", 5, 2)
+    out, dx, grads = U.hip_run(mod, x, g, hip_device, dtype=torch.float16, param_dtype=torch.float16)
+    assert all(p.grad.dtype == torch.float16 for p in mod.parameters() if p.grad is not None)
+    wo, wdx, wg = U.oracle_run(ref, x, g, torch.float64)
+
+    def close16(a, b, name):
+        rms = b.double().pow(2).mean().sqrt().item()
+        torch.testing.assert_close(a.double(), b.double(), rtol=2e-3, atol=2e-3 * rms, msg=lambda m: f"{name}: {m}")
+    close16(out, wo, "out")
+    close16(dx, wdx, "grad_x")
+    for n, v in grads.items():
+        close16(v, wg[n], n)
 
 
 def test_fp16_under_autocast(hip_device):

@@ -14,6 +14,10 @@ def _bf16_round(a):
     return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).to(torch.float32).numpy()
 
 
+def _f16_round(a):
+    return np.ascontiguousarray(a).astype(np.float16).astype(np.float32)
+
+
 def _case2d(B, C, H, W, K, L, bias, dtype=0, pdtype=0, seed=0):
     rng = np.random.default_rng(seed)
     f = lambda *s: rng.standard_normal(s).astype(np.float32)
@@ -22,11 +26,13 @@ def _case2d(B, C, H, W, K, L, bias, dtype=0, pdtype=0, seed=0):
     ws = [f(4 * C, 1, K, K) * 0.3 for _ in range(L)]
     ss = [f(1, 4 * C, 1, 1) for _ in range(L)]
     if dtype:
-        x, g = _bf16_round(x), _bf16_round(g)
+        rd = _f16_round if dtype == 2 else _bf16_round
+        x, g = rd(x), rd(g)
     if pdtype:
-        bw, bs = _bf16_round(bw), _bf16_round(bs)
-        bb = _bf16_round(bb) if bias else None
-        ws, ss = [_bf16_round(w) for w in ws], [_bf16_round(s) for s in ss]
+        rd = _f16_round if pdtype == 2 else _bf16_round
+        bw, bs = rd(bw), rd(bs)
+        bb = rd(bb) if bias else None
+        ws, ss = [rd(w) for w in ws], [rd(s) for s in ss]
     return x, g, bw, bb, bs, ws, ss
 
 
@@ -46,11 +52,14 @@ def _oracle(dims, x, g, bw, bb, bs, ws, ss):
     return res
 
 
-def _compare(got, want, rtol, atol_scale):
-    def chk(a, b, name):
+def _compare(got, want, rtol, atol_scale, act_tol=None):
+    """`act_tol`: its own (rtol, atol_scale) for the two activation-typed results, out and dx."""
+    def chk(a, b, name, rt=rtol, at=atol_scale):
         scale = max(float(np.sqrt(np.mean(b.astype(np.float64) ** 2))), 1e-6)
-        np.testing.assert_allclose(a, b, rtol=rtol, atol=atol_scale * scale, err_msg=name)
-    for k in ("out", "dx", "dbase_w", "dbase_s"):
+        np.testing.assert_allclose(a, b, rtol=rt, atol=at * scale, err_msg=name)
+    for k in ("out", "dx"):
+        chk(got[k], want[k], k, *(act_tol or (rtol, atol_scale)))
+    for k in ("dbase_w", "dbase_s"):
         chk(got[k], want[k], k)
     if "dbase_b" in want:
         chk(got["dbase_b"], want["dbase_b"], "dbase_b")
@@ -180,6 +189,40 @@ def test_emulated_2d_bf16_io_and_params():
     _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-2, atol_scale=2e-2)
 
 
+@pytest.mark.parametrize("B,C,H,W,K,L,bias,pdtype", [
+    (1, 2, 8, 12, 5, 2, True, 2),      # rows of whole 4-element vectors, half parameters
+    (2, 1, 9, 7, 3, 2, True, 0),       # odd sizes: element-wise loads and stores
+    (1, 1, 24, 40, 7, 3, False, 0),
+    (1, 1, 300, 280, 5, 2, True, 0),   # level-by-level kernels (plane beyond LDS)
+])
+def test_emulated_2d_fp16(B, C, H, W, K, L, bias, pdtype):
+    """IEEE half tensors: the vector-ALU kernels read and write them and compute in fp32, so the outputs differ from
+    the oracle by their final rounding (2^-11 relative) and the parameter gradients hold the fp32 bar."""
+    x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias, dtype=2, pdtype=pdtype)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, K, dtype=2, pdtype=pdtype)
+    want = _oracle(2, x, g, bw, bb, bs, ws, ss)
+    # half parameters get their gradients as fp32 as well: the fp32 bar either way
+    _compare(got, want, rtol=2e-5, atol_scale=2e-5, act_tol=(1e-3, 1e-3))
+
+
+def test_emulated_half_conversions():
+    """The emulation's own half <-> float conversions against numpy's, over every half bit pattern and a float sweep
+    that crosses the subnormal, normal and overflow ranges (the GPU uses the hardware conversion instead)."""
+    h = np.arange(65536, dtype=np.uint16)
+    vals = h.view(np.float16).astype(np.float32)
+    finite = np.isfinite(vals)
+    got = emu_util.half_roundtrip(vals[finite])
+    np.testing.assert_array_equal(got.view(np.uint32), vals[finite].view(np.uint32))
+    rng = np.random.default_rng(5)
+    f = (rng.standard_normal(20000) * np.exp(rng.uniform(-20, 12, 20000))).astype(np.float32)
+    f = np.concatenate([f, np.float32([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 2.0 ** -24, 2.0 ** -25,
+                                       1.5 * 2.0 ** -25, 6.1e-5, 6.0e-5])])
+    got = emu_util.half_roundtrip(f)
+    with np.errstate(over="ignore"):
+        want = f.astype(np.float16).astype(np.float32)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_emulated_2d_stage1_plane():
     """One plane of the WTConvNeXt-T stage-1 shape (56x56, K=5, L=3)."""
     x, g, bw, bb, bs, ws, ss = _case2d(1, 1, 56, 56, 5, 3, True)
@@ -212,6 +255,15 @@ def test_emulated_1d_fp32(B, C, N, K, L, bias):
     x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, bias)
     got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K)
     _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
+
+
+@pytest.mark.parametrize("B,C,N,K,L", [(2, 2, 1000, 5, 4), (1, 2, 517, 5, 3), (1, 1, 37, 3, 3), (1, 1, 17000, 5, 4)])
+def test_emulated_1d_fp16(B, C, N, K, L):
+    x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, True)
+    x, g = _f16_round(x), _f16_round(g)
+    got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K, dtype=2)
+    want = _oracle(1, x, g, bw, bb, bs, ws, ss)
+    _compare(got, want, rtol=2e-5, atol_scale=2e-5, act_tol=(1e-3, 1e-3))
 
 
 def test_emulated_1d_row_resident_bf16():

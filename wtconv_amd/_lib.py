@@ -6,9 +6,9 @@ import threading
 from . import _build
 
 MAX_LEVELS = 5
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 PASS_FORWARD, PASS_BACKWARD_INPUT, PASS_BACKWARD_PARAMS, PASS_BACKWARD = 0, 1, 2, 3
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Params(ctypes.Structure):

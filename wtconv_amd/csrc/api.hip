@@ -16,6 +16,14 @@
 
 namespace wt {
 
+// The element type of the activations as the template argument `T_` of a launcher call.
+#define WT_BY_DTYPE(dtype, CALL)                                              \
+  ((dtype) == WTCONV_F32 ? [&] { using T_ = float; return CALL; }()          \
+   : (dtype) == WTCONV_BF16 ? [&] { using T_ = bf16_t; return CALL; }()      \
+                            : [&] { using T_ = f16_t; return CALL; }())
+
+static inline bool known_dtype(int d) { return d == WTCONV_F32 || d == WTCONV_BF16 || d == WTCONV_F16; }
+
 static int check_common(const char* fn, const wtconv_params* params, int B, int C, int K, int L,
                         int dtype, int pdtype) {
   if (B <= 0 || C <= 0) return fail(WTCONV_E_ARG, "%s: batch and channels must be positive (got %d, %d)", fn, B, C);
@@ -24,8 +32,8 @@ static int check_common(const char* fn, const wtconv_params* params, int B, int 
     return fail(WTCONV_E_UNSUPPORTED, "%s: kernel_size %d exceeds the largest built kernel (%d)", fn, K,
                 wtconv_max_kernel_size());
   if (L < 1 || L > kMaxLevels) return fail(WTCONV_E_ARG, "%s: wt_levels must be 1-%d (got %d)", fn, kMaxLevels, L);
-  if (dtype != WTCONV_F32 && dtype != WTCONV_BF16) return fail(WTCONV_E_ARG, "%s: unknown dtype %d", fn, dtype);
-  if (pdtype != WTCONV_F32 && pdtype != WTCONV_BF16) return fail(WTCONV_E_ARG, "%s: unknown param dtype %d", fn, pdtype);
+  if (!known_dtype(dtype)) return fail(WTCONV_E_ARG, "%s: unknown dtype %d", fn, dtype);
+  if (!known_dtype(pdtype)) return fail(WTCONV_E_ARG, "%s: unknown param dtype %d", fn, pdtype);
   if (params == nullptr || params->base_weight == nullptr || params->base_scale == nullptr)
     return fail(WTCONV_E_ARG, "%s: null parameter pointer", fn);
   for (int l = 0; l < L; ++l)
@@ -369,8 +377,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
     float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
     float* pyr = fw + round_up64(fold_floats(C, 4, L, K * K));
     if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
-    return dtype == WTCONV_F32 ? run_stream2d_k<float>(K, x, out, fw, fb, pyr, sp, stream)
-                               : run_stream2d_k<bf16_t>(K, x, out, fw, fb, pyr, sp, stream);
+    return WT_BY_DTYPE(dtype, run_stream2d_k<T_>(K, x, out, fw, fb, pyr, sp, stream));
   }
   Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
   int tj1 = 4, sg_shift = 8;
@@ -385,12 +392,12 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
-  if (dtype == WTCONV_F32) {
-    const int e = run_plane2d_static<float>(K, tj1, x, out, fw, fb, pl, stream);
+  if (dtype != WTCONV_BF16) {     // (bf16 tensors of these shapes are on the matrix-core kernels)
+    const int e = dtype == WTCONV_F32 ? run_plane2d_static<float>(K, tj1, x, out, fw, fb, pl, stream)
+                                      : run_plane2d_static<f16_t>(K, tj1, x, out, fw, fb, pl, stream);
     if (e != 1) return e;
   }
-  return dtype == WTCONV_F32 ? run_plane2d_k<float>(K, tj1, x, out, fw, fb, pl, stream)
-                             : run_plane2d_k<bf16_t>(K, tj1, x, out, fw, fb, pl, stream);
+  return WT_BY_DTYPE(dtype, run_plane2d_k<T_>(K, tj1, x, out, fw, fb, pl, stream));
 }
 
 // ---- 1-D dispatch -------------------------------------------------------------------
@@ -584,11 +591,9 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
   if (int e = launch_fold(params, pdtype, fw, fb, C, 2, L, K, flip, flip ? 0 : 1, stream)) return e;
   if (row_resident) {
     const Row1D rp = make_row1d(C, N, nl, esz, x, out);
-    return dtype == WTCONV_F32 ? run_row1d_kl<float>(K, L, x, out, fw, fb, rp, B, block, stream)
-                               : run_row1d_kl<bf16_t>(K, L, x, out, fw, fb, rp, B, block, stream);
+    return WT_BY_DTYPE(dtype, run_row1d_kl<T_>(K, L, x, out, fw, fb, rp, B, block, stream));
   }
-  return dtype == WTCONV_F32 ? run_tile1d_k<float>(K, x, out, fw, fb, pl, B, stream)
-                             : run_tile1d_k<bf16_t>(K, x, out, fw, fb, pl, B, stream);
+  return WT_BY_DTYPE(dtype, run_tile1d_k<T_>(K, x, out, fw, fb, pl, B, stream));
 }
 
 // ---- static scratch for callers that may not allocate ------------------------------------
@@ -740,19 +745,18 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
     Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
     finish_wgrad_plan(&pl, K);
     wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
-    e = dtype == WTCONV_F32 ? run_wgrad2d_static<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream) : 1;
+    e = dtype == WTCONV_F32   ? run_wgrad2d_static<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+        : dtype == WTCONV_F16 ? run_wgrad2d_static<f16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+                              : 1;
     if (e == 1)
-      e = dtype == WTCONV_F32 ? run_wgrad2d_k<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
-                              : run_wgrad2d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream);
+      e = WT_BY_DTYPE(dtype, run_wgrad2d_k<T_>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream));
   } else {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     nchunk = stream_chunks(B, C, H, W);
     if (nchunk > 65535 || C > 0x7fffffff / 4) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
     float* pyr_x = partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * L) * K * K + 1));
     float* pyr_g = pyr_x + sp.floats;
-    e = dtype == WTCONV_F32
-            ? run_stream2d_wgrad_k<float>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream)
-            : run_stream2d_wgrad_k<bf16_t>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
+    e = WT_BY_DTYPE(dtype, run_stream2d_wgrad_k<T_>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream));
   }
   if (e) return e;
   GradTable gt = {};
@@ -847,13 +851,9 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   int e;
   if (row_resident) {
     const Row1D rp = make_row1d(C, N, nl, esz, x, grad_out);
-    e = dtype == WTCONV_F32
-            ? run_row1d_wgrad_kl<float>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream)
-            : run_row1d_wgrad_kl<bf16_t>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream);
+    e = WT_BY_DTYPE(dtype, run_row1d_wgrad_kl<T_>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream));
   } else {
-    e = dtype == WTCONV_F32
-            ? run_wgrad1d_k<float>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream)
-            : run_wgrad1d_k<bf16_t>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream);
+    e = WT_BY_DTYPE(dtype, run_wgrad1d_k<T_>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream));
   }
   if (e) return e;
   GradTable gt = {};

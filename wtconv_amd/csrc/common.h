@@ -118,18 +118,83 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 #endif
 
+// IEEE half storage: a type of its own, so that templates tell it from bf16.  The vector-ALU kernels read and write
+// it and compute in fp32 (haar_common.cuh:55-77 of the reference dispatches the same three element types).
+struct f16_t { uint16_t bits; };
+
+#ifdef WT_EMULATE
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  const uint32_t ex = (h >> 10) & 31u, man = h & 0x3ffu;
+  if (ex == 31u) return __uint_as_float(sign | 0x7f800000u | (man << 13));
+  if (ex == 0u) {                                        // zero and subnormals: man * 2^-24, exact in fp32
+    const float v = static_cast<float>(man) * 5.9604644775390625e-8f;
+    return sign ? -v : v;
+  }
+  return __uint_as_float(sign | ((ex + 112u) << 23) | (man << 13));
+}
+// round-to-nearest-even, overflow to infinity, NaN kept quiet
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint16_t sign = static_cast<uint16_t>((u >> 16) & 0x8000u);
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return static_cast<uint16_t>(sign | 0x7e00u);
+  if (a >= 0x477ff000u) return static_cast<uint16_t>(sign | 0x7c00u);      // >= 65520 rounds to infinity
+  if (a < 0x33000001u) return sign;                                        // <= 2^-25 rounds to zero
+  const int e = static_cast<int>(a >> 23) - 127;
+  uint32_t man = (a & 0x7fffffu) | 0x800000u;                              // 24 significant bits
+  const int shift = e >= -14 ? 13 : 13 + (-14 - e);                        // bits dropped (subnormals drop more)
+  const uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  uint32_t r = kept + ((rest > half || (rest == half && (kept & 1u))) ? 1u : 0u);
+  // normal: r holds the implicit one at bit 10, so adding the biased exponent - 1 carries correctly on mantissa overflow
+  const uint32_t bits = e >= -14 ? (static_cast<uint32_t>(e + 14) << 10) + r : r;
+  return static_cast<uint16_t>(sign | bits);
+}
+#else
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+#endif
+
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+template <> __device__ __forceinline__ float to_f32<f16_t>(f16_t v) { return f16_bits_to_f32(v.bits); }
 
 template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return f16_t{f32_to_f16_bits(v)}; }
+
+// Two 16-bit elements of type T in one 32-bit word (the first in the low half): unpack to fp32, pack from fp32.
+template <typename T> __device__ __forceinline__ void unpack2(uint32_t w, float& lo, float& hi);
+template <> __device__ __forceinline__ void unpack2<bf16_t>(uint32_t w, float& lo, float& hi) {
+  lo = __uint_as_float(w << 16); hi = __uint_as_float(w & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t w, float& lo, float& hi) {
+  lo = f16_bits_to_f32(static_cast<uint16_t>(w)); hi = f16_bits_to_f32(static_cast<uint16_t>(w >> 16));
+}
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
+#ifdef WT_EMULATE
+  return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
+#else
+  typedef float wt_f32x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 wt_f16x2 __attribute__((ext_vector_type(2)));
+  const wt_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, wt_f16x2));
+#endif
+}
 
 // parameter fetch with a run-time dtype (only used while folding parameters)
 __device__ __forceinline__ float load_param(const void* p, int dtype, int idx) {
-  return dtype == WTCONV_F32 ? static_cast<const float*>(p)[idx]
-                             : bf16_to_f32(static_cast<const bf16_t*>(p)[idx]);
+  if (dtype == WTCONV_F32) return static_cast<const float*>(p)[idx];
+  const uint16_t h = static_cast<const uint16_t*>(p)[idx];
+  return dtype == WTCONV_F16 ? f16_bits_to_f32(h) : bf16_to_f32(h);
 }
 
 // Kernel-argument copy of wtconv_params.

@@ -56,8 +56,7 @@ __device__ __forceinline__ void load_row_tile(const T* __restrict__ row, float* 
           const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            vals[2 * k] = __uint_as_float(qq[k] << 16);
-            vals[2 * k + 1] = __uint_as_float(qq[k] & 0xffff0000u);
+            unpack2<T>(qq[k], vals[2 * k], vals[2 * k + 1]);
           }
         }
       } else {
@@ -113,10 +112,10 @@ __device__ __forceinline__ void store_run(T* __restrict__ dst, const float (&v)[
 #pragma unroll
       for (int k = 0; k < N / 8; ++k) {
         uint4 q;
-        q.x = pack_bf16x2(v[8 * k], v[8 * k + 1]);
-        q.y = pack_bf16x2(v[8 * k + 2], v[8 * k + 3]);
-        q.z = pack_bf16x2(v[8 * k + 4], v[8 * k + 5]);
-        q.w = pack_bf16x2(v[8 * k + 6], v[8 * k + 7]);
+        q.x = pack2<T>(v[8 * k], v[8 * k + 1]);
+        q.y = pack2<T>(v[8 * k + 2], v[8 * k + 3]);
+        q.z = pack2<T>(v[8 * k + 4], v[8 * k + 5]);
+        q.w = pack2<T>(v[8 * k + 6], v[8 * k + 7]);
         reinterpret_cast<uint4*>(dst)[k] = q;
       }
     }

@@ -108,8 +108,7 @@ __device__ __forceinline__ void row1d_commit(float* __restrict__ lds, int nl, in
         const uint32_t qq[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          vals[2 * k] = __uint_as_float(qq[k] << 16);
-          vals[2 * k + 1] = __uint_as_float(qq[k] & 0xffff0000u);
+          unpack2<T>(qq[k], vals[2 * k], vals[2 * k + 1]);
         }
       }
       row1d_put<S, SLOT, EV>(lds, p, vals);
@@ -135,8 +134,7 @@ __device__ __forceinline__ void row1d_stage_pair(const T* __restrict__ row0, con
       const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        vals[2 * k] = __uint_as_float(qq[k] << 16);
-        vals[2 * k + 1] = __uint_as_float(qq[k] & 0xffff0000u);
+        unpack2<T>(qq[k], vals[2 * k], vals[2 * k + 1]);
       }
     }
   };
@@ -205,7 +203,7 @@ __device__ __forceinline__ void row1d_unstage(T* __restrict__ row, const float* 
         uint32_t qq[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          qq[k] = pack_bf16x2(vals[2 * k], vals[2 * k + 1]);
+          qq[k] = pack2<T>(vals[2 * k], vals[2 * k + 1]);
         q.x = qq[0]; q.y = qq[1]; q.z = qq[2]; q.w = qq[3];
       }
       *reinterpret_cast<uint4*>(row + p) = q;

@@ -126,8 +126,8 @@ __device__ __forceinline__ void load4(const T* __restrict__ p, float (&v)[4]) {
     v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
   } else {
     const uint2 q = *reinterpret_cast<const uint2*>(p);
-    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
-    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+    unpack2<T>(q.x, v[0], v[1]);
+    unpack2<T>(q.y, v[2], v[3]);
   }
 }
 
@@ -526,8 +526,8 @@ __device__ __forceinline__ void store_row(T* __restrict__ dst, const float (&v)[
           *reinterpret_cast<float4*>(dst + 4 * k) = q;
         } else {
           uint2 q;
-          q.x = pack_bf16x2(v[4 * k], v[4 * k + 1]);
-          q.y = pack_bf16x2(v[4 * k + 2], v[4 * k + 3]);
+          q.x = pack2<T>(v[4 * k], v[4 * k + 1]);
+          q.y = pack2<T>(v[4 * k + 2], v[4 * k + 3]);
           *reinterpret_cast<uint2*>(dst + 4 * k) = q;
         }
       }

@@ -292,9 +292,12 @@ __device__ __forceinline__ void fold_entry(const ParamTable& p, int pdtype, int 
 #pragma unroll
       for (int i = 0; i < 5; ++i) wr[i] = w[i < K ? i : K - 1];
     } else {
-      const bf16_t* w = static_cast<const bf16_t*>(wp) + rowi;
+      const uint16_t* w = static_cast<const uint16_t*>(wp) + rowi;
+      uint16_t h[5];
 #pragma unroll
-      for (int i = 0; i < 5; ++i) wr[i] = bf16_to_f32(w[i < K ? i : K - 1]);
+      for (int i = 0; i < 5; ++i) h[i] = w[i < K ? i : K - 1];
+#pragma unroll
+      for (int i = 0; i < 5; ++i) wr[i] = pdtype == WTCONV_F16 ? f16_bits_to_f32(h[i]) : bf16_to_f32(h[i]);
     }
     if (row_ok) {
 #pragma unroll

@@ -174,7 +174,7 @@ Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype) {
   Mfma2dQuery r = {false, 0};
   const int mode = mfma_mode();
   if (mode <= 0 || K > 5 || L < 1 || L > kMaxLevels) return r;
-  if (dtype == WTCONV_F32 && mode < 2) return r;
+  if (dtype != WTCONV_BF16 && !(dtype == WTCONV_F32 && mode >= 2)) return r;
   const int NS = dtype == WTCONV_F32 ? 3 : 1;
   MPlan pl;
   int nbl;

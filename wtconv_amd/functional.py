@@ -11,7 +11,7 @@ import torch
 
 from . import _lib
 
-_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
 
 
 def check_kernel_size(kernel_size):
@@ -31,7 +31,7 @@ def _ptr(t):
 
 
 def _prep_params(x, base_w, base_b, base_s, wt_ws, wt_ss):
-    """Contiguous parameter tensors in one dtype the kernels accept (fp32 or bf16)."""
+    """Contiguous parameter tensors in one dtype the kernels accept (fp32, bf16 or fp16)."""
     tensors = [base_w, base_s] + list(wt_ws) + list(wt_ss) + ([base_b] if base_b is not None else [])
     pd = base_w.dtype
     if pd not in _DT or any(t.dtype != pd for t in tensors):
@@ -89,7 +89,7 @@ def _check_input(x, ndim, what):
         raise ValueError(f"{what} expects a {ndim}-D input, got shape {tuple(x.shape)}")
     if not x.is_cuda:
         raise RuntimeError(f"{what} runs on the GPU only (got a {x.device} tensor); there is no CPU path")
-    if x.dtype not in _DT and x.dtype != torch.float16:
+    if x.dtype not in _DT:
         raise TypeError(f"{what} supports float32, bfloat16 and float16 activations, got {x.dtype}")
 
 
@@ -132,12 +132,8 @@ def _forward_impl(x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L, tabinfo=N
     lib = _lib.load()
     if not x.is_contiguous():
         x = x.contiguous()
-    if x.dtype == torch.float16:
-        # float16 activations (the reference trainer's default AMP dtype, train.py:180,438; its
-        # fused twin dispatches fp16 too, haar_common.cuh:55-77) are widened at the boundary: the
-        # fp32 kernels run on the exact fp16 values and the result is rounded to fp16 once.
-        out, _ = _forward_impl(x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L)
-        return out.to(torch.float16), x
+    # float16 activations (the reference trainer's default AMP dtype, train.py:180,438; its fused twin dispatches
+    # fp16 too, haar_common.cuh:55-77) go through the vector kernels: fp16 in HBM, fp32 arithmetic, one rounding.
     pd, tab, _keep = _params_table(x, base_w, base_b, base_s, wt_ws, wt_ss)
     if tabinfo is not None:
         tabinfo.append((pd, tab, _keep))
@@ -160,10 +156,6 @@ def _backward_impl(grad_out, x, base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L
     base_s, wt_ws[0..L-1], wt_ss[0..L-1] (all None when not needed), in the parameters' dtypes."""
     lib = _lib.load()
     g = grad_out
-    if x.dtype == torch.float16:          # widened at the boundary, as in the forward pass
-        grad_x, grads = _backward_impl(g.float(), x.float(), base_w, base_b, base_s, wt_ws, wt_ss, dims, K, L,
-                                       need_x, need_params)
-        return (grad_x.to(torch.float16) if grad_x is not None else None), grads
     if g.dtype != x.dtype:
         g = g.to(x.dtype)
     if not g.is_contiguous():
@@ -237,8 +229,8 @@ class _WTConvFn(torch.autograd.Function):
     """dims = 2: x (B,C,H,W); dims = 1: x (B,C,N).  Argument order:
     x, base_w, base_b, base_s, dims, K, L, wt_w[0..L-1], wt_s[0..L-1]."""
 
-    # Under torch.autocast the inputs are taken as they come (fp32 or bf16 activations, fp32 or
-    # bf16 parameters, any mix): the kernels accumulate in fp32 either way, so there is nothing
+    # Under torch.autocast the inputs are taken as they come (fp32, bf16 or fp16 activations, parameters in any of
+    # the three, any mix): the kernels accumulate in fp32 either way, so there is nothing
     # to down-cast, and neither pass runs a torch operator that autocast would touch (hence no
     # custom_fwd / custom_bwd wrappers: entering an autocast context costs more host time than the
     # rest of the backward prelude).
@@ -247,7 +239,7 @@ class _WTConvFn(torch.autograd.Function):
         info = []
         out, x = _forward_impl(x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L, info)
         ctx.dims, ctx.K, ctx.L = dims, K, L
-        ctx.tabinfo = info[0] if info and x.dtype != torch.float16 else None
+        ctx.tabinfo = info[0] if info else None
         ctx.save_for_backward(x, base_w, base_b, base_s, *wt)
         return out
 
