@@ -319,8 +319,49 @@ def bench_model(torch, dev, steps, warmup, batch=256):
     x = torch.randn(batch, 3, 224, 224, device=dev).bfloat16()
     with torch.no_grad():
         wall_ms, med_ms, _, _ = time_steps(torch, lambda i: model(x), 1, steps, warmup)
-    return {"workload": f"WTConvNeXt-T bf16 inference forward, batch {batch}, 3x224x224, WTConv layers on the HIP kernels",
-            "ms_per_step": wall_ms, "images_per_s": batch / (wall_ms * 1e-3)}
+    res = {"workload": f"WTConvNeXt-T bf16 inference forward, batch {batch}, 3x224x224, WTConv layers on the HIP kernels",
+           "ms_per_step": wall_ms, "images_per_s": batch / (wall_ms * 1e-3)}
+    gms = model_graph_ms(torch, model, x, steps, warmup)
+    if gms is not None:
+        res["hip_graph_replay"] = {"ms_per_step": gms, "images_per_s": batch / (gms * 1e-3)}
+    return res
+
+
+def model_graph_ms(torch, model, x, steps, warmup):
+    """The same forward captured in one HIP graph.  Library calls inside the model (convolutions, GEMMs, the
+    mean) are captured as they come, so every replay is checked against the eager logits, with eager work and a
+    synchronisation between replays, before the replay time is reported; None if the capture fails or differs."""
+    try:
+        with torch.no_grad():
+            want = model(x).float()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                model(x)
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=side):
+                    out = model(x)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            for _ in range(3):
+                out.zero_()
+                gr.replay()
+                torch.cuda.synchronize()
+                if not torch.equal(out.float(), want):
+                    return None
+                model(x)                                  # eager work between the replays
+                torch.cuda.synchronize()
+            for _ in range(warmup):
+                gr.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                gr.replay()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps * 1e3
+    except Exception as e:      # capture is an extra; the eager figure above is the measurement
+        print(f"bench.py: model graph capture failed: {e}", file=sys.stderr)
+        return None
 
 
 def cpu_baseline(torch, workload, cpu_batch):
