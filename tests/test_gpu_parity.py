@@ -658,6 +658,61 @@ def test_config4_full_size_1d(hip_device):
     _full_size_properties("1d", 64, 5, 4, (64, 64, 4096), hip_device, torch.float32)
 
 
+@pytest.mark.parametrize("kind,dtype", [("2d", torch.bfloat16), ("2d", torch.float32), ("1d", torch.float32)])
+def test_tensor_beyond_2_31_elements(hip_device, kind, dtype):
+    """Tensors of more than 2^31 elements (element offsets need 64 bits): the input and the upstream gradient are zero
+    except in a few batch items at both ends and in the middle.  Those items must come out bit-identical to the layer run
+    on them alone (a plane's arithmetic does not depend on where it sits), the parameter gradients equal to that small
+    run's up to the order of the fp32 chunk sums."""
+    W2, W1 = _mods()
+    free, _ = torch.cuda.mem_get_info()
+    esz = 2 if dtype == torch.bfloat16 else 4
+    if free < 5 * (2 ** 31 + 2 ** 27) * esz:
+        pytest.skip("not enough free device memory for four tensors of 2^31 elements")
+    if kind == "2d":
+        C, K, L, tail = 8, 5, 3, (56, 56)
+        B = 2 ** 31 // (C * 56 * 56) + 40
+        mod = W2(C, C, K, wt_levels=L)
+    else:
+        C, K, L, tail = 16, 5, 4, (4096,)
+        B = 2 ** 31 // (C * 4096) + 24
+        mod = W1(C, C, K, wt_levels=L)
+    torch.manual_seed(11)
+    U.randomize_scales(mod, seed=4)
+    mod = mod.to(hip_device)
+    if dtype == torch.bfloat16:
+        mod = mod.to(dtype)
+    sel = [0, 1, B // 2, B - 2, B - 1]
+    xs = torch.randn(len(sel), C, *tail).to(device=hip_device, dtype=dtype)
+    gs = torch.randn(len(sel), C, *tail).to(device=hip_device, dtype=dtype)
+    assert B * C * xs[0, 0].numel() > 2 ** 31
+
+    def run(x, g):
+        for p in mod.parameters():
+            p.grad = None
+        x = x.requires_grad_(True)
+        out = mod(x)
+        out.backward(g)
+        torch.cuda.synchronize()
+        return out.detach(), x.grad, [p.grad.float().clone() for p in mod.parameters() if p.grad is not None]
+
+    so, sdx, sgr = run(xs.clone(), gs)
+    x = torch.zeros(B, C, *tail, device=hip_device, dtype=dtype)
+    g = torch.zeros(B, C, *tail, device=hip_device, dtype=dtype)
+    x[sel] = xs
+    g[sel] = gs
+    out, dx, gr = run(x, g)
+    assert torch.equal(out[sel], so), "outputs of the selected batch items"
+    assert torch.equal(dx[sel], sdx), "input gradients of the selected batch items"
+    # a batch item in between, where x and the upstream gradient are zero: the bias path alone, no input gradient
+    assert torch.equal(out[B // 3], out[B // 3 + 1]) and not dx[B // 3].any()
+    for a, b_ in zip(gr, sgr):
+        if dtype == torch.bfloat16:
+            torch.testing.assert_close(a, b_, rtol=2e-2, atol=2e-2 * max(b_.abs().max().item(), 1e-6))
+        else:
+            torch.testing.assert_close(a, b_, rtol=1e-5, atol=1e-4)
+
+
 # ------------------------------------------------------------------ caller harness
 def test_wtconvnext_harness_hip_vs_oracle_conv_class(hip_device):
     """WTConvNeXt-T (reduced depth) with the HIP WTConv2d against the same host model with the
