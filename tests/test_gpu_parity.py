@@ -406,6 +406,46 @@ def test_torch_compile_against_oracle(hip_device):
     U.compare_all((oc.detach().cpu(), xc.grad.cpu(), grads), U.oracle_run(ref, x, g, torch.float64), U.assert_fp32)
 
 
+def test_torch_compile_inductor_against_oracle(hip_device):
+    """backend="inductor" (the default of the reference's trainer, train.py:629-632): generated pointwise kernels
+    around the opaque layer operator, forward and every gradient against the CPU oracle wrapped the same way."""
+    W2, _ = _mods()
+    ref, x, g = U.seeded_case("2d", 6, 5, 2, (2, 6, 20, 24))
+    U.randomize_scales(ref)
+
+    class Net(torch.nn.Module):
+        def __init__(self, conv):
+            super().__init__()
+            self.conv = conv
+
+        def forward(self, t):
+            return torch.nn.functional.gelu(self.conv(t) * 2 + t)
+
+    net = Net(U.copy_to_hip_module(ref, W2, "2d", 5, 2)).to(hip_device)
+    try:
+        cnet = torch.compile(net, backend="inductor", fullgraph=True)
+        xc = x.to(hip_device).requires_grad_(True)
+        oc = cnet(xc)
+    except Exception as e:      # no usable code generator on this machine
+        if "inductor" in repr(e).lower() or "triton" in repr(e).lower():
+            pytest.skip(f"inductor backend not usable here: {type(e).__name__}")
+        raise
+    oc.backward(g.to(hip_device))
+    torch.cuda.synchronize()
+    rnet = Net(ref).double()
+    xr = x.double().requires_grad_(True)
+    orf = rnet(xr)
+    orf.backward(g.double())
+    U.assert_fp32(oc.detach().cpu(), orf.detach(), "out")
+    U.assert_fp32(xc.grad.cpu(), xr.grad, "grad_x")
+    want = {n: p.grad for n, p in rnet.named_parameters() if p.grad is not None}
+    got = {n: p.grad.detach().cpu() for n, p in net.named_parameters() if p.grad is not None}
+    trainable = [n for n in want if "wt_filter" not in n]
+    assert set(trainable) <= set(got)
+    for n in trainable:
+        U.assert_fp32(got[n], want[n], n)
+
+
 def test_gradient_checkpointing(hip_device):
     """torch.utils.checkpoint around the layer (WTConvNeXt stages offer it, wtconvnext.py:209-210 of the
     reference): the recomputed forward and the backward through it match the oracle."""
