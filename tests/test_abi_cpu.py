@@ -187,3 +187,21 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setenv("WTCONV_HIP_LIB", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.WTConvLibraryError, match="no fallback"):
         _lib.load()
+
+
+def test_cpp_autograd_node_builds_loads_and_declines_host_tensors(lib):
+    """The C++ autograd node (host code only) compiles against the installed PyTorch, takes the library's entry
+    points by address, and hands anything that is not a GPU tensor in a kernel dtype back to the Python path."""
+    from wtconv_amd import _build, _ext
+    if (not os.path.exists(_build.BINDING_PATH)
+            or os.path.getmtime(_build.BINDING_PATH) < os.path.getmtime(_build.BINDING_SRC)):
+        _build.build_binding()
+        _ext._tried, _ext._mod = False, None
+    ext = _ext.get()
+    assert ext is not None
+    C, K = 4, 3
+    x = torch.randn(1, C, 8, 8)
+    args = (torch.randn(C, 1, K, K), torch.randn(C), torch.randn(1, C, 1, 1), [torch.randn(4 * C, 1, K, K)],
+            [torch.randn(1, 4 * C, 1, 1)])
+    assert ext.layer(x, *args, 2, K, 1) is None
+    assert ext.layer(x, args[0], None, *args[2:], 2, K, 1) is None

@@ -1,4 +1,5 @@
-"""Builds libwtconv_hip.so in-tree with hipcc for gfx950 (no JIT, no cache directory)."""
+"""Builds libwtconv_hip.so in-tree with hipcc for gfx950, and the C++ autograd node that PyTorch calls it through
+(no JIT, no cache directory)."""
 import os
 import subprocess
 
@@ -53,6 +54,36 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
+BINDING_SRC = os.path.join(CSRC, "torch_binding.cpp")
+BINDING_NAME = "_wtconv_torch"
+BINDING_PATH = os.path.join(PKG_DIR, BINDING_NAME + ".so")
+
+
+def build_binding(verbose=False):
+    """Compile the C++ autograd node (host code only: g++ against the headers of the installed PyTorch).  It calls
+    the HIP library through addresses handed over at import, so it links against PyTorch alone."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-w",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1", f"-DTORCH_EXTENSION_NAME={BINDING_NAME}",
+           "-DTORCH_API_INCLUDE_EXTENSION_H"]
+    cmd += ["-I" + p for p in cpp_extension.include_paths()]
+    cmd += ["-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(rocm, "include")]
+    cmd += [BINDING_SRC, "-o", BINDING_PATH + ".tmp", "-L" + tlib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+            "-ltorch_python"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the PyTorch binding failed:\n" + r.stdout[-4000:] + r.stderr[-8000:])
+    os.replace(BINDING_PATH + ".tmp", BINDING_PATH)
+    return BINDING_PATH
+
+
 def is_stale():
     if not os.path.exists(LIB_PATH):
         return True
@@ -62,3 +93,4 @@ def is_stale():
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_binding(verbose=True))

@@ -9,7 +9,7 @@ from typing import List, Optional
 
 import torch
 
-from . import _lib
+from . import _ext, _lib
 
 _DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
 
@@ -312,6 +312,13 @@ _op_forward.register_autograd(_op_autograd_backward, setup_context=_op_setup_con
 def _apply(x, base_weight, base_bias, base_scale, wt_weights, wt_scales, dims, K, L):
     if torch.compiler.is_compiling():
         return _op_forward(x, base_weight, base_bias, base_scale, list(wt_weights), list(wt_scales), dims)
+    ext = _ext.get()
+    if ext is not None:
+        # the same launches from a C++ autograd node (no interpreter between PyTorch's engine and the library);
+        # None: parameters that need a conversion first (mixed dtypes, another device, not contiguous)
+        out = ext.layer(x, base_weight, base_bias, base_scale, list(wt_weights), list(wt_scales), dims, K, L)
+        if out is not None:
+            return out
     return _WTConvFn.apply(x, base_weight, base_bias, base_scale, dims, K, L, *wt_weights, *wt_scales)
 
 
