@@ -61,6 +61,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary dtype and per-kernel timing")
     ap.add_argument("--cpu-batch", type=int, default=16)
+    ap.add_argument("--settle", type=float, default=SETTLE_SECONDS,
+                    help="seconds of untimed work before each timed leg, for the GPU to reach its running clocks "
+                         "(0 for counter-collection runs, where every launch is slow)")
     ap.add_argument("--only-1d", action="store_true",
                     help="run only the WTConv1d(64,64,5,wt_levels=4) x[64,64,4096] workload and print its line")
     ap.add_argument("--only-model", action="store_true",
@@ -87,18 +90,53 @@ def make_sets(torch, dev, dtype, C, H, W, B, nsets):
     return sets
 
 
+SETTLE_SECONDS = 0.15
+
+
+def settle(torch, fn, nsets, seconds=None):
+    """Runs the workload for `seconds` before any warm-up or timing: after an idle spell (set-up, a capture, the
+    synchronisation behind the previous leg) the GPU takes some tens of milliseconds of work to reach its running
+    clocks -- measured on this layer: the first 25 steps after idle average 0.49 ms, the next 25 0.44 ms, every later
+    one 0.420 ms -- and a training loop runs in that last state."""
+    seconds = SETTLE_SECONDS if seconds is None else seconds
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn(i % nsets)
+            i += 1
+        torch.cuda.synchronize()
+
+
 def time_steps(torch, fn, nsets, steps, warmup):
+    """(wall ms per step over exactly `steps` steps between two synchronisations; median, min, mean of the per-step
+    HIP-event times of a pass of `steps` steps before it).  The wall-clock pass holds nothing but the steps: the
+    interpreter's cyclic garbage collector is off while it runs (as in `timeit`; a collection over the objects of
+    the earlier legs costs milliseconds, i.e. whole steps of a sub-millisecond workload), and the per-step events
+    are recorded in a pass of their own."""
+    import gc
+    gc.collect()
+    settle(torch, fn, nsets)
     for i in range(warmup):
         fn(i % nsets)
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    t0 = time.perf_counter()
-    for i in range(steps):
-        evs[i][0].record()
-        fn(i % nsets)
-        evs[i][1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i in range(steps):
+            evs[i][0].record()
+            fn(i % nsets)
+            evs[i][1].record()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i % nsets)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    finally:
+        if was_on:
+            gc.enable()
     per = [a.elapsed_time(b) for a, b in evs]         # ms, HIP events on the launch stream
     return wall / steps * 1e3, statistics.median(per), min(per), sum(per) / len(per)
 
@@ -131,6 +169,7 @@ def graph_step_ms(torch, mod, sets, steps, warmup):
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         n = len(graphs)
+        settle(torch, lambda i: graphs[i][0].replay(), n)
         for i in range(warmup):
             graphs[i % n][0].replay()
         torch.cuda.synchronize()
@@ -351,6 +390,7 @@ def model_graph_ms(torch, model, x, steps, warmup):
                     return None
                 model(x)                                  # eager work between the replays
                 torch.cuda.synchronize()
+            settle(torch, lambda i: gr.replay(), 1)
             for _ in range(warmup):
                 gr.replay()
             torch.cuda.synchronize()
@@ -433,6 +473,8 @@ def roofline_of(ks, workload, dtype, K, L, P):
 
 def main():
     args = parse()
+    global SETTLE_SECONDS
+    SETTLE_SECONDS = max(0.0, args.settle)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); the layer is data-parallel per "
               "plane and no multi-GPU figure is produced", file=sys.stderr)
@@ -469,7 +511,7 @@ def main():
         "metric": "WTConv2d fwd+bwd images/s",
         "value": main_res["images_per_s"],
         "unit": "images/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_s": SETTLE_SECONDS,
         "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"fp32": "f32", "bf16": "bf16", "fp16": "f16 in HBM, f32 arithmetic"}[args.dtype],

@@ -127,7 +127,7 @@ def test_stage_shapes_bf16_small_batch(hip_device, C, H, L, bf16_params):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_stage_planes_at_the_batch_of_their_compile_time_plans(hip_device, B, H, L, dtype):
     """The four stage plane sizes with enough batch items that the kernels take the planes-per-unit of their
-    compile-time plans (1, 4, 11, 29 forward; 1, 3, 12, 24 and 1, 3, 12, 16 for the gradients), few channels:
+    compile-time plans (1, 4, 11, 29 forward; 1, 2, 7, 16 for the gradients), few channels:
     every output and gradient against the oracle."""
     W2, _ = _mods()
     C = 4

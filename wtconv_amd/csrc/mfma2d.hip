@@ -204,6 +204,7 @@ int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* p
 namespace {
 
 constexpr int kWgradLdsPair = 80 * 1024;      // two workgroups of four waves per CU below this, else one of eight waves
+constexpr int kWgradLdsTriple = 53 * 1024;    // three workgroups per CU below this
 
 struct WKey {
   int B, C, H, W, L;
@@ -218,8 +219,11 @@ struct WKeyHash {
 };
 struct WVal { bool ok; WPlan pl; int nw, compact, bchunk, nchunk; };
 
-// Planes per unit: up to one 4x4 block per thread of four waves, within the LDS that leaves room for two
-// workgroups per CU; a single plane beyond that runs as one workgroup of eight waves per CU.
+// Planes per unit: up to one 4x4 block per thread of four waves.  Small planes, of which at least two fit a third
+// of the LDS, run as three workgroups per CU (a unit's phases are short and wait on its loads, so a third
+// workgroup in another phase pays more than larger units: 7 x 7 planes 38 -> 28 us, 14 x 14 34 -> 29 us, 28 x 28
+// 57 -> 50 us per launch at batch 128); otherwise as many planes as leave room for two workgroups per CU; a single
+// plane beyond that runs as one workgroup of eight waves per CU.
 bool choose_wplan(int B, int C, int H, int W, int L, WVal* v) {
   const int bpp0 = ceil_div(H, 4) * ceil_div(W, 4);
   int pb = kMfmaBlock / bpp0;
@@ -228,9 +232,16 @@ bool choose_wplan(int B, int C, int H, int W, int L, WVal* v) {
   if (static_cast<long long>(pb) * C * H * W > 0x7fffffffLL) return false;
   WPlan pl;
   bool compact = false;
+  const int pb_max = pb;
   for (;; --pb) {
     if (!make_wplan_geometry(H, W, L, pb, 512, false, &pl)) return false;
-    if (pl.lds_bytes <= kWgradLdsPair || pb == 1) break;
+    if (pl.lds_bytes <= kWgradLdsTriple || pb == 1) break;
+  }
+  if (pl.lds_bytes > kWgradLdsTriple || (pb < 2 && pb_max >= 2)) {
+    for (pb = pb_max;; --pb) {
+      if (!make_wplan_geometry(H, W, L, pb, 512, false, &pl)) return false;
+      if (pl.lds_bytes <= kWgradLdsPair || pb == 1) break;
+    }
   }
   if (pl.lds_bytes > kWgradLdsPair) {
     WPlan cp;
@@ -241,7 +252,8 @@ bool choose_wplan(int B, int C, int H, int W, int L, WVal* v) {
   v->pl = pl;
   v->compact = compact;
   v->nw = pl.lds_bytes <= kWgradLdsPair ? 4 : 8;
-  wgrad_chunks(B, C, pb, compute_units() * (v->nw == 4 ? 2 : 1), &v->bchunk, &v->nchunk);
+  const int per_cu = v->nw == 8 ? 1 : (pl.lds_bytes <= kWgradLdsTriple ? 3 : 2);
+  wgrad_chunks(B, C, pb, compute_units() * per_cu, &v->bchunk, &v->nchunk);
   return true;
 }
 
@@ -278,8 +290,8 @@ int launch_wgrad_l(int nw, bool compact, bool vec, const WgradArgs& a, const WPl
 #define WT_TRY(H_, L_, PB_, NW_, CMP_) \
   if (L == L_ && pl.H == H_ && pl.W == H_ && pl.pb == PB_ && nw == NW_ && compact == CMP_ && vec == (H_ % 4 == 0)) \
     return launch_wgrad<L_, NW_, H_ % 4 == 0, WGeoStatic<H_, H_, L_, PB_, 512, CMP_>>(a, pl, stream);
-  WT_TRY(56, 3, 1, 4, true) WT_TRY(28, 3, 3, 4, false) WT_TRY(14, 2, 12, 4, false) WT_TRY(7, 2, 24, 4, false)
-  WT_TRY(56, 5, 1, 8, false) WT_TRY(28, 4, 2, 4, false) WT_TRY(14, 3, 8, 4, false)
+  WT_TRY(56, 3, 1, 4, true) WT_TRY(28, 3, 2, 4, false) WT_TRY(14, 2, 7, 4, false) WT_TRY(7, 2, 16, 4, false)
+  WT_TRY(56, 5, 1, 8, false) WT_TRY(28, 4, 2, 4, false) WT_TRY(14, 3, 4, 4, false)
 #undef WT_TRY
 #endif
   if (vec)
