@@ -22,6 +22,9 @@ namespace wt {
    : (dtype) == WTCONV_BF16 ? [&] { using T_ = bf16_t; return CALL; }()      \
                             : [&] { using T_ = f16_t; return CALL; }())
 
+// Threads of wgrad_finish_kernel: one per entry of a channel's record (taps of every filter + sumG) where that fits.
+static inline int finish_threads(int nrec) { return nrec >= 1024 ? 1024 : (nrec + kWave - 1) / kWave * kWave; }
+
 static inline bool known_dtype(int d) { return d == WTCONV_F32 || d == WTCONV_BF16 || d == WTCONV_F16; }
 
 static int check_common(const char* fn, const wtconv_params* params, int B, int C, int K, int L,
@@ -765,7 +768,7 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   gt.base_scale = grads->base_scale;
   for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
   const int nrec = (1 + 4 * L) * K * K + 1;
-  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(256), static_cast<size_t>(nrec) * sizeof(float),
+  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(finish_threads(nrec)), static_cast<size_t>(nrec) * sizeof(float),
             stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 4, L, K * K);
   return check_launch("wgrad_finish_kernel");
 }
@@ -862,7 +865,7 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   gt.base_scale = grads->base_scale;
   for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
   const int nrec = (1 + 2 * L) * K + 1;
-  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(256), static_cast<size_t>(nrec) * sizeof(float),
+  WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(finish_threads(nrec)), static_cast<size_t>(nrec) * sizeof(float),
             stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 2, L, K);
   return check_launch("wgrad_finish_kernel");
 }

@@ -1076,31 +1076,32 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
 // Second stage: sum the per-chunk partials and apply the chain rule of the folding
 //   dw = gamma * dWt,  dgamma = sum_t w * dWt (+ bias * sumG for the base scale),
 //   dbias = gamma_b * sumG        (cf. fast_wtconv/cuda_haar/haar_cuda.py:168-197,657-676)
-// One workgroup per channel, one thread per (filter, tap); the per-filter dot products go
-// through LDS.  S = 4 (2-D) or 2 (1-D).  blockDim.x >= NF, dynamic LDS NF*KK floats.
+// One workgroup per channel, one thread per (filter, tap) plus one for sumG (a single pass when the workgroup has
+// NF*KK + 1 threads: the kernel is a chain of load latencies, nothing else); the per-filter dot products go
+// through LDS.  S = 4 (2-D) or 2 (1-D).  blockDim.x >= NF, dynamic LDS NF*KK + 1 floats.
 __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchunk, ParamTable p,
                                     int pdtype, GradTable gt, int C, int S, int L, int KK) {
   WT_SHARED_FLOATS(prod);
   const int NF = 1 + S * L;
   const int stride = NF * KK + 1;
   const int c = blockIdx.x;
-  for (int o = threadIdx.x; o < NF * KK; o += blockDim.x) {
+  for (int o = threadIdx.x; o <= NF * KK; o += blockDim.x) {      // (the last index is the sumG slot of the records)
+    const bool tap = o < NF * KK;
+    const int f = tap ? o / KK : 0, t = tap ? o - f * KK : 0;
+    const int l = f == 0 ? 0 : (f - 1) / S, chn = f == 0 ? c : c * S + (f - 1) % S;
+    // parameters first: their loads overlap those of the partial sums
+    const float gam = load_param(f == 0 ? p.base_scale : p.wt_scale[l], pdtype, chn);
+    const float wv = load_param(f == 0 ? p.base_weight : p.wt_weight[l], pdtype, chn * KK + t);
     float sum = 0.f;
 #pragma unroll 8                       // several chunk loads in flight; the order of the adds is unchanged
     for (int ch = 0; ch < nchunk; ++ch) sum += partial[(static_cast<size_t>(ch) * C + c) * stride + o];
-    const int f = o / KK, t = o - f * KK;
-    float gam, wv;
-    if (f == 0) {
-      gam = load_param(p.base_scale, pdtype, c);
-      wv = load_param(p.base_weight, pdtype, c * KK + t);
-      gt.base_weight[c * KK + t] = gam * sum;
+    if (tap) {
+      float* dst = f == 0 ? gt.base_weight : gt.wt_weight[l];
+      dst[chn * KK + t] = gam * sum;
+      prod[o] = wv * sum;
     } else {
-      const int l = (f - 1) / S, chn = c * S + (f - 1) % S;
-      gam = load_param(p.wt_scale[l], pdtype, chn);
-      wv = load_param(p.wt_weight[l], pdtype, chn * KK + t);
-      gt.wt_weight[l][chn * KK + t] = gam * sum;
+      prod[o] = sum;
     }
-    prod[o] = wv * sum;
   }
   const int o = threadIdx.x;
   __syncthreads();
@@ -1108,10 +1109,7 @@ __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchun
     float dot = 0.f;
     for (int t = 0; t < KK; ++t) dot += prod[o * KK + t];
     if (o == 0) {
-      // sumG sits in the last slot of the channel's partial record
-      float sg = 0.f;
-#pragma unroll 8
-      for (int ch = 0; ch < nchunk; ++ch) sg += partial[(static_cast<size_t>(ch) * C + c) * stride + NF * KK];
+      const float sg = prod[NF * KK];
       if (p.base_bias != nullptr) {
         dot = fmaf(load_param(p.base_bias, pdtype, c), sg, dot);
         if (gt.base_bias != nullptr) gt.base_bias[c] = load_param(p.base_scale, pdtype, c) * sg;
