@@ -11,18 +11,22 @@
 namespace wt {
 namespace {
 
-// Largest power-of-two pixel tile (8..64) whose [C][tp + 1] floats, plus the per-pixel statistics, stay within
-// 48 KB of LDS (three workgroups per CU); false if even 8 pixels do not fit or the sizes overflow the indexing.
-bool make_block_tile(int C, int HW, BlockTile* out, size_t* lds_bytes) {
+// Largest power-of-two pixel tile (8..64) whose [C][tp + 1] elements of `esz` bytes, plus the per-pixel statistics,
+// stay within 48 KB of LDS (three workgroups per CU); false if even 8 pixels do not fit or the sizes overflow the
+// indexing.
+bool make_block_tile(int C, int HW, size_t esz, BlockTile* out, size_t* lds_bytes) {
   BlockTile t = {};
   t.C = C; t.HW = HW;
   int tp = 64;
-  // tile, two sets of partial sums [256 / p][p], mean and rstd [2][p], weight and bias [2][C]
-  auto bytes = [&](int p) { return (static_cast<size_t>(C) * (p + 1) + 2 * kBlockThreads + 2 * p + 2 * static_cast<size_t>(C)) * sizeof(float); };
+  // tile (rounded up to 16 bytes), then floats: two sets of partial sums [256 / p][p], mean and rstd [2][p],
+  // weight and bias [2][C]
+  auto tile_bytes = [&](int p) { return (static_cast<size_t>(C) * (p + 1) * esz + 15) / 16 * 16; };
+  auto bytes = [&](int p) { return tile_bytes(p) + (2 * kBlockThreads + 2 * p + 2 * static_cast<size_t>(C)) * sizeof(float); };
   while (tp > 8 && bytes(tp) > 48 * 1024) tp >>= 1;
   if (bytes(tp) > kLdsLimitBytes) return false;
   while (tp > 8 && tp / 2 >= HW) tp >>= 1;          // tiny images: no lanes without a pixel
   t.tp = tp;
+  t.aux = static_cast<int>(tile_bytes(tp) / sizeof(float));
   t.tp_shift = 0;
   while ((1 << t.tp_shift) < tp) ++t.tp_shift;
   t.tiles = (HW + tp - 1) / tp;
@@ -38,35 +42,45 @@ bool make_block_tile(int C, int HW, BlockTile* out, size_t* lds_bytes) {
 }
 
 struct TileKey {
-  int C, HW;
-  bool operator==(const TileKey& o) const { return C == o.C && HW == o.HW; }
+  int C, HW, esz;
+  bool operator==(const TileKey& o) const { return C == o.C && HW == o.HW && esz == o.esz; }
 };
 struct TileKeyHash {
-  size_t operator()(const TileKey& k) const { return (static_cast<size_t>(k.C) << 32) ^ static_cast<size_t>(k.HW); }
+  size_t operator()(const TileKey& k) const {
+    return (static_cast<size_t>(k.C) << 32) ^ (static_cast<size_t>(k.HW) << 3) ^ static_cast<size_t>(k.esz);
+  }
 };
-struct TileVal { bool ok; BlockTile t; size_t lds; };
+struct TileVal { bool ok; BlockTile t; size_t lds; int esz; };      // esz: bytes of a tile element
 
-const TileVal& block_tile_cached(int C, int HW) {
+const TileVal& block_tile_cached(int C, int HW, int esz) {
   static thread_local std::unordered_map<TileKey, TileVal, TileKeyHash> cache;
-  const TileKey key = {C, HW};
+  const TileKey key = {C, HW, esz};
   auto it = cache.find(key);
   if (it == cache.end()) {
     if (cache.size() > 4096) cache.clear();
     TileVal v = {};
-    v.ok = make_block_tile(C, HW, &v.t, &v.lds);
+    v.ok = make_block_tile(C, HW, static_cast<size_t>(esz), &v.t, &v.lds);
+    v.esz = esz;
     it = cache.emplace(key, v).first;
   }
   return it->second;
 }
 
-int check_block_args(const char* fn, int B, int C, int HW, int dtype, int pdtype, const TileVal** tv) {
+// float_tile: the caller can keep bf16 tensors as floats in LDS; taken where that still gives 64 pixels per tile.
+int check_block_args(const char* fn, int B, int C, int HW, int dtype, int pdtype, const TileVal** tv,
+                     bool float_tile = false) {
   if (B <= 0 || C <= 0 || HW <= 0) return fail(WTCONV_E_ARG, "%s: sizes must be positive (got B=%d C=%d HW=%d)", fn, B, C, HW);
   if (C % 2) return fail(WTCONV_E_UNSUPPORTED, "%s: the channel count must be even (got %d)", fn, C);
   if ((dtype != WTCONV_F32 && dtype != WTCONV_BF16) || (pdtype != WTCONV_F32 && pdtype != WTCONV_BF16))
     return fail(WTCONV_E_ARG, "%s: unknown dtype code", fn);
   if (B > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: batch %d exceeds the launch grid", fn, B);
   if (static_cast<long long>(C) * HW > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "%s: an image of %d x %d elements is too large", fn, C, HW);
-  const TileVal& v = block_tile_cached(C, HW);
+  const TileVal* vp = &block_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2);
+  if (float_tile && dtype != WTCONV_F32) {
+    const TileVal& vf = block_tile_cached(C, HW, 4);
+    if (vf.ok && vf.t.tp == 64) vp = &vf;
+  }
+  const TileVal& v = *vp;
   if (!v.ok) return fail(WTCONV_E_UNSUPPORTED, "%s: %d channels do not fit a tile in LDS", fn, C);
   *tv = &v;
   return 0;
@@ -81,7 +95,7 @@ extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight,
                                    float eps, int dtype, int param_dtype, int out_nhwc, void* stream_) {
   const char* fn = "wtconv_channel_norm";
   const TileVal* tv = nullptr;
-  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv)) return e;
+  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv, true)) return e;
   if (x == nullptr || out == nullptr || weight == nullptr || bias == nullptr) return fail(WTCONV_E_ARG, "%s: null pointer", fn);
   if (x == out) return fail(WTCONV_E_ARG, "%s: in-place use is not supported (tiles of the output overlap other tiles' input)", fn);
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
@@ -99,10 +113,13 @@ extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight,
     return check_launch("channel_norm_kernel");
   };
   if (dtype == WTCONV_F32)
-    return vec ? launch(channel_norm_kernel<float, true>, static_cast<float*>(nullptr))
-               : launch(channel_norm_kernel<float, false>, static_cast<float*>(nullptr));
-  return vec ? launch(channel_norm_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
-             : launch(channel_norm_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+    return vec ? launch(channel_norm_kernel<float, float, true>, static_cast<float*>(nullptr))
+               : launch(channel_norm_kernel<float, float, false>, static_cast<float*>(nullptr));
+  if (tv->esz == 4)      // bf16 tensor, tile of floats
+    return vec ? launch(channel_norm_kernel<bf16_t, float, true>, static_cast<bf16_t*>(nullptr))
+               : launch(channel_norm_kernel<bf16_t, float, false>, static_cast<bf16_t*>(nullptr));
+  return vec ? launch(channel_norm_kernel<bf16_t, bf16_t, true>, static_cast<bf16_t*>(nullptr))
+             : launch(channel_norm_kernel<bf16_t, bf16_t, false>, static_cast<bf16_t*>(nullptr));
 }
 
 extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const void* gamma, void* out, int B, int C,

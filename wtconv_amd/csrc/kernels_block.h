@@ -4,11 +4,15 @@
 // trips through HBM, two of them layout copies; here each side is one kernel that transposes through LDS:
 //   channel_norm_kernel    NCHW -> LayerNorm over C -> NHWC (or NCHW: the LayerNorm2d of stem and downsample layers)
 //   block_residual_kernel  NHWC y, NCHW shortcut -> shortcut + gamma[c] * y, NCHW
-// A workgroup takes a tile of TP consecutive pixels of one image with all their channels: [C][TP + 1] floats in
-// LDS (the odd row pitch keeps both the pixel-major and the channel-major sweep free of bank conflicts).  The
-// NCHW side moves TP contiguous elements per channel, the NHWC side the tile's TP * C elements, which are one
-// contiguous run.  Statistics are two sweeps over LDS in fp32 (mean, then the sum of squared deviations).
+// A workgroup takes a tile of TP consecutive pixels of one image with all their channels: [C][TP + 1] elements in
+// LDS, in the tensors' own element type (the values pass through unchanged; bf16 tiles are half the size, so twice
+// the pixels fit: longer contiguous runs on the NCHW side and more workgroups per CU).  The odd row pitch keeps
+// both the pixel-major and the channel-major sweep free of bank conflicts.  The NCHW side moves TP contiguous
+// elements per channel, the NHWC side the tile's TP * C elements, which are one contiguous run.  Statistics are
+// two sweeps over LDS in fp32 (mean, then the sum of squared deviations).
 #pragma once
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -18,7 +22,8 @@ constexpr int kBlockThreads = 256;
 
 struct BlockTile {
   int C, HW;
-  int tp;            // pixels per tile: a power of two, 8..64
+  int tp;            // pixels per tile: a power of two, 8..128
+  int aux;           // float index in LDS where the arrays behind the tile start
   int tp_shift;
   int tiles;         // tiles per image
   unsigned mg_c;     // reciprocal of C for dividends < tp * C (shift 32)
@@ -40,6 +45,17 @@ template <> __device__ __forceinline__ void store_pair<float>(float* p, float a,
 template <> __device__ __forceinline__ void store_pair<bf16_t>(bf16_t* p, float a, float b) {
   *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(a, b);
 }
+// two consecutive elements as they are
+template <typename T>
+__device__ __forceinline__ void load_pair_raw(const T* p, T& a, T& b);
+template <> __device__ __forceinline__ void load_pair_raw<float>(const float* p, float& a, float& b) {
+  const float2 v = *reinterpret_cast<const float2*>(p);
+  a = v.x; b = v.y;
+}
+template <> __device__ __forceinline__ void load_pair_raw<bf16_t>(const bf16_t* p, bf16_t& a, bf16_t& b) {
+  const uint32_t v = *reinterpret_cast<const uint32_t*>(p);
+  a = static_cast<bf16_t>(v); b = static_cast<bf16_t>(v >> 16);
+}
 template <typename T>
 __device__ __forceinline__ void load_pair(const T* p, float& a, float& b);
 template <> __device__ __forceinline__ void load_pair<float>(const float* p, float& a, float& b) {
@@ -57,6 +73,7 @@ template <> struct Quad<float> {
   float4 v;
   __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
   __device__ __forceinline__ void get(float (&f)[4]) const { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
+  __device__ __forceinline__ void raw(float (&f)[4]) const { get(f); }
 };
 template <> struct Quad<bf16_t> {
   uint2 v;
@@ -65,14 +82,21 @@ template <> struct Quad<bf16_t> {
     f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
     f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
   }
+  __device__ __forceinline__ void raw(bf16_t (&f)[4]) const {
+    f[0] = static_cast<bf16_t>(v.x); f[1] = static_cast<bf16_t>(v.x >> 16);
+    f[2] = static_cast<bf16_t>(v.y); f[3] = static_cast<bf16_t>(v.y >> 16);
+  }
 };
 
 constexpr int kQuadBatch = 6;      // vector loads a thread keeps in flight before it writes them to LDS
 
-// NCHW tile -> LDS [C][tp + 1]; pixels past the image are left alone (never read back).
+// tile element from / to fp32 (LT = float or the tensor's type)
+template <typename LT> __device__ __forceinline__ float tile_get(LT v) { return to_f32<LT>(v); }
+
+// NCHW tile -> LDS [C][tp + 1] of LT (float, or T itself); pixels past the image are left alone (never read back).
 // VEC: HW is a multiple of 4 and the tensor 4-element aligned, so rows move as 4-element vectors.
-template <typename T, bool VEC>
-__device__ __forceinline__ void tile_from_nchw(const T* __restrict__ img, float* lds, const BlockTile& t, int p0, int tid) {
+template <typename T, typename LT, bool VEC>
+__device__ __forceinline__ void tile_from_nchw(const T* __restrict__ img, LT* lds, const BlockTile& t, int p0, int tid) {
   const int pitch = t.tp + 1;
   if constexpr (VEC) {
     const int gshift = t.tp_shift - 2;                       // 4-pixel groups per tile row
@@ -91,8 +115,9 @@ __device__ __forceinline__ void tile_from_nchw(const T* __restrict__ img, float*
         for (int k = 0; k < kQuadBatch; ++k) {
           const int c = cb + k * cstep;
           if (c < t.C) {
-            float f[4];
-            q[k].get(f);
+            LT f[4];
+            if constexpr (std::is_same<LT, T>::value) q[k].raw(f);
+            else q[k].get(f);
 #pragma unroll
             for (int j = 0; j < 4; ++j) lds[c * pitch + p + j] = f[j];
           }
@@ -102,26 +127,32 @@ __device__ __forceinline__ void tile_from_nchw(const T* __restrict__ img, float*
   } else {
     const int p = tid & (t.tp - 1), c0 = tid >> t.tp_shift, cstep = kBlockThreads >> t.tp_shift;
     if (p0 + p < t.HW)
-      for (int c = c0; c < t.C; c += cstep) lds[c * pitch + p] = to_f32<T>(img[static_cast<size_t>(c) * t.HW + p0 + p]);
+      for (int c = c0; c < t.C; c += cstep) {
+        const T v = img[static_cast<size_t>(c) * t.HW + p0 + p];
+        if constexpr (std::is_same<LT, T>::value) lds[c * pitch + p] = v;
+        else lds[c * pitch + p] = to_f32<T>(v);
+      }
   }
 }
 
-// Grid (tiles, B).  out_nhwc != 0: out is (B, HW, C); else (B, C, HW).
-template <typename T, bool VEC>
+// Grid (tiles, B).  out_nhwc != 0: out is (B, HW, C); else (B, C, HW).  LT: the tile's element type -- fp32 where
+// that reaches 64 pixels per tile (the three sweeps over the tile then cost no conversions), else T.
+template <typename T, typename LT, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __restrict__ weight,
                     const void* __restrict__ bias, int pdtype, float eps, int out_nhwc, const BlockTile t) {
-  WT_SHARED_FLOATS(lds);
+  WT_SHARED_FLOATS(ldsf);
+  LT* lds = reinterpret_cast<LT*>(ldsf);         // the tile
   const int tid = threadIdx.x;
   const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
   const int pitch = t.tp + 1, C = t.C;
   const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
-  float* psum = lds + C * pitch;                 // [parts][tp] partial sums
+  float* psum = ldsf + t.aux;                    // [parts][tp] partial sums
   float* pvar = psum + kBlockThreads;            // [parts][tp] partial sums of squared deviations
   float* stat = pvar + kBlockThreads;            // mean[tp], rstd[tp]
   float* wgt = stat + 2 * t.tp;                  // weight[C], bias[C]
   const T* img = x + static_cast<size_t>(b) * C * t.HW;
-  tile_from_nchw<T, VEC>(img, lds, t, p0, tid);
+  tile_from_nchw<T, LT, VEC>(img, lds, t, p0, tid);
   for (int c = tid; c < C; c += kBlockThreads) {
     wgt[c] = load_param(weight, pdtype, c);
     wgt[C + c] = load_param(bias, pdtype, c);
@@ -131,7 +162,7 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
   const bool live = p < np;
   float s = 0.f;
   if (live)
-    for (int c = part_i; c < C; c += parts) s += lds[c * pitch + p];
+    for (int c = part_i; c < C; c += parts) s += tile_get<LT>(lds[c * pitch + p]);
   psum[part_i * t.tp + p] = s;
   __syncthreads();
   float mean = 0.f;
@@ -140,7 +171,7 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
   float v = 0.f;
   if (live)
     for (int c = part_i; c < C; c += parts) {
-      const float d = lds[c * pitch + p] - mean;
+      const float d = tile_get<LT>(lds[c * pitch + p]) - mean;
       v += d * d;
     }
   pvar[part_i * t.tp + p] = v;
@@ -158,15 +189,15 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
       const int e = 2 * i;
       const int pp = div_c(e, t.mg_c), c = e - pp * C;
       const float m = stat[pp], r = stat[t.tp + pp];
-      const float a = (lds[c * pitch + pp] - m) * r * wgt[c] + wgt[C + c];
-      const float bb = (lds[(c + 1) * pitch + pp] - m) * r * wgt[c + 1] + wgt[C + c + 1];
+      const float a = (tile_get<LT>(lds[c * pitch + pp]) - m) * r * wgt[c] + wgt[C + c];
+      const float bb = (tile_get<LT>(lds[(c + 1) * pitch + pp]) - m) * r * wgt[c + 1] + wgt[C + c + 1];
       store_pair<T>(dst + e, a, bb);
     }
   } else {
     T* dst = out + static_cast<size_t>(b) * C * t.HW + p0;
     if (live)
       for (int c = part_i; c < C; c += parts)
-        dst[static_cast<size_t>(c) * t.HW + p] = from_f32<T>((lds[c * pitch + p] - mean) * rstd * wgt[c] + wgt[C + c]);
+        dst[static_cast<size_t>(c) * t.HW + p] = from_f32<T>((tile_get<LT>(lds[c * pitch + p]) - mean) * rstd * wgt[c] + wgt[C + c]);
   }
 }
 
@@ -175,7 +206,8 @@ template <typename T, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, const void* __restrict__ gamma,
                       int pdtype, T* __restrict__ out, const BlockTile t) {
-  WT_SHARED_FLOATS(lds);
+  WT_SHARED_FLOATS(ldsf);
+  T* lds = reinterpret_cast<T*>(ldsf);
   const int tid = threadIdx.x;
   const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
   const int pitch = t.tp + 1, C = t.C;
@@ -185,8 +217,8 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
   for (int i = tid; i < npair; i += kBlockThreads) {
     const int e = 2 * i;
     const int pp = div_c(e, t.mg_c), c = e - pp * C;
-    float a, bb;
-    load_pair<T>(src + e, a, bb);
+    T a, bb;
+    load_pair_raw<T>(src + e, a, bb);
     lds[c * pitch + pp] = a;
     lds[(c + 1) * pitch + pp] = bb;
   }
@@ -212,8 +244,9 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
             float f[4];
             q[k].get(f);
             T* o = out + base + static_cast<size_t>(c) * t.HW;
-            store_pair<T>(o, f[0] + gm * lds[c * pitch + p], f[1] + gm * lds[c * pitch + p + 1]);
-            store_pair<T>(o + 2, f[2] + gm * lds[c * pitch + p + 2], f[3] + gm * lds[c * pitch + p + 3]);
+            const T* row = lds + c * pitch + p;
+            store_pair<T>(o, f[0] + gm * to_f32<T>(row[0]), f[1] + gm * to_f32<T>(row[1]));
+            store_pair<T>(o + 2, f[2] + gm * to_f32<T>(row[2]), f[3] + gm * to_f32<T>(row[3]));
           }
         }
       }
@@ -225,7 +258,7 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
       for (int c = c0; c < C; c += cstep) {
         const float g = gamma != nullptr ? load_param(gamma, pdtype, c) : 1.f;
         const size_t o = base + static_cast<size_t>(c) * t.HW;
-        out[o] = from_f32<T>(to_f32<T>(shortcut[o]) + g * lds[c * pitch + p]);
+        out[o] = from_f32<T>(to_f32<T>(shortcut[o]) + g * to_f32<T>(lds[c * pitch + p]));
       }
     }
   }
