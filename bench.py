@@ -324,7 +324,7 @@ def bench_1d(torch, dev, steps, warmup):
     gtab = Fn._table(_lib.ParamGrads, f32(bw), f32(bb), f32(bs), [f32(w) for w in ws], [f32(s_) for s_ in ss])
     outs = [torch.empty_like(sets[i][0]) for i in range(nsets)]
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    wsz = max(lib.wtconv1d_workspace_bytes(B, C, N, K, L, p) for p in (0, 1, 2))
+    wsz = max(lib.wtconv1d_workspace_bytes(B, C, N, K, L, p) for p in (0, 1, 2, 3))
     wsp = torch.empty(wsz, dtype=torch.uint8, device=dev)
     P_ = Fn._ptr
 
@@ -340,12 +340,19 @@ def bench_1d(torch, dev, steps, warmup):
         assert lib.wtconv1d_backward_params(P_(sets[i][0]), P_(sets[i][1]), ctypes.byref(tab), ctypes.byref(gtab),
                                             B, C, N, K, L, 0, 0, P_(wsp), wsz, stream) == 0, lib.wtconv_last_error()
 
+    gxs = [torch.empty_like(sets[i][0]) for i in range(nsets)]
+
+    def k_bwd(i):      # the whole backward pass as the module's autograd node calls it: one fused kernel
+        assert lib.wtconv1d_backward(P_(sets[i][0]), P_(sets[i][1]), P_(gxs[i]), ctypes.byref(tab), ctypes.byref(gtab),
+                                     B, C, N, K, L, 0, 0, P_(wsp), wsz, stream) == 0, lib.wtconv_last_error()
+
     kern = {}
-    for name, fn in (("wt1d_row_kernel(forward)", k_fwd), ("wt1d_row_kernel(backward_input)", k_bwd_in),
-                     ("wt1d_row_wgrad_kernel", k_bwd_par)):
+    for name, fn, nbytes in (("wt1d_row_kernel(forward)", k_fwd, 2), ("wt1d_row_kernel(backward_input)", k_bwd_in, 2),
+                             ("wt1d_row_wgrad_kernel", k_bwd_par, 2), ("wt1d_row_bwd_kernel(backward)", k_bwd, 3)):
         _, med, mn, avg = time_steps(torch, fn, nsets, steps, warmup)
-        kern[name] = {"avg_ms": avg, "median_ms": med, "min_ms": mn, "algorithmic_bytes": 2 * P * 4,
-                      "GBps": 2 * P * 4 / (avg * 1e-3) / 1e9, "frac_hbm": 2 * P * 4 / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        kern[name] = {"avg_ms": avg, "median_ms": med, "min_ms": mn, "algorithmic_bytes": nbytes * P * 4,
+                      "GBps": nbytes * P * 4 / (avg * 1e-3) / 1e9,
+                      "frac_hbm": nbytes * P * 4 / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     res["kernels"] = kern
     return res
 

@@ -102,7 +102,9 @@ int wtconv2d_forward(const void* x, void* out, const wtconv_params* params,
  * a pyramid in the workspace) are rejected with WTCONV_E_UNSUPPORTED.  The call allocates and
  * frees nothing.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
  * (two streams, two threads) race; calls on one stream are ordered and safe.  The result is
- * bit-identical to wtconv2d_forward. */
+ * bit-identical to wtconv2d_forward.  The first call on a GPU looks up the address of that GPU's
+ * array (hipGetDevice + hipGetSymbolAddress, under a mutex) and must therefore happen outside a
+ * stream capture; every later call on that GPU only launches kernels and may be captured. */
 size_t wtconv_static_scratch_bytes(void);
 
 int wtconv2d_forward_static(const void* x, void* out, const wtconv_params* params,

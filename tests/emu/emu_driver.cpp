@@ -105,28 +105,42 @@ int main(int argc, char** argv) {
   for (int l = 0; l < L; ++l) { gr.wt_weight[l] = dws[l].data(); gr.wt_scale[l] = dss[l].data(); }
 
   int rc = 0;
+  const char* fused_env = getenv("WT_EMU_FUSED_BWD");      // "1": the whole backward pass through wtconv*_backward
+  const bool fused = fused_env != nullptr && fused_env[0] == '1';
   auto ws_alloc = [&](size_t bytes) { return std::vector<char>(bytes); };   // exact size: ASan guards it
   if (dims == 2) {
     auto w0 = ws_alloc(wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_FORWARD));
     rc = wtconv2d_forward(x.ptr(), out.ptr(), &prm, B, C, H, W, K, L, dtype, pdtype, w0.data(), w0.size(), nullptr);
     if (rc) { fprintf(stderr, "forward: %s\n", wtconv_last_error()); return 3; }
+    if (fused) {
+      auto w3 = ws_alloc(wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD));
+      rc = wtconv2d_backward(x.ptr(), g.ptr(), dx.ptr(), &prm, &gr, B, C, H, W, K, L, dtype, pdtype, w3.data(), w3.size(), nullptr);
+      if (rc) { fprintf(stderr, "backward: %s\n", wtconv_last_error()); return 3; }
+    } else {
     auto w1 = ws_alloc(wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD_INPUT));
     rc = wtconv2d_backward_input(g.ptr(), dx.ptr(), &prm, B, C, H, W, K, L, dtype, pdtype, w1.data(), w1.size(), nullptr);
     if (rc) { fprintf(stderr, "backward_input: %s\n", wtconv_last_error()); return 3; }
     auto w2 = ws_alloc(wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD_PARAMS));
     rc = wtconv2d_backward_params(x.ptr(), g.ptr(), &prm, &gr, B, C, H, W, K, L, dtype, pdtype, w2.data(), w2.size(), nullptr);
     if (rc) { fprintf(stderr, "backward_params: %s\n", wtconv_last_error()); return 3; }
+    }
   } else {
     const int N = W;
     auto w0 = ws_alloc(wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_FORWARD));
     rc = wtconv1d_forward(x.ptr(), out.ptr(), &prm, B, C, N, K, L, dtype, pdtype, w0.data(), w0.size(), nullptr);
     if (rc) { fprintf(stderr, "forward: %s\n", wtconv_last_error()); return 3; }
+    if (fused) {
+      auto w3 = ws_alloc(wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_BACKWARD));
+      rc = wtconv1d_backward(x.ptr(), g.ptr(), dx.ptr(), &prm, &gr, B, C, N, K, L, dtype, pdtype, w3.data(), w3.size(), nullptr);
+      if (rc) { fprintf(stderr, "backward: %s\n", wtconv_last_error()); return 3; }
+    } else {
     auto w1 = ws_alloc(wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_BACKWARD_INPUT));
     rc = wtconv1d_backward_input(g.ptr(), dx.ptr(), &prm, B, C, N, K, L, dtype, pdtype, w1.data(), w1.size(), nullptr);
     if (rc) { fprintf(stderr, "backward_input: %s\n", wtconv_last_error()); return 3; }
     auto w2 = ws_alloc(wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_BACKWARD_PARAMS));
     rc = wtconv1d_backward_params(x.ptr(), g.ptr(), &prm, &gr, B, C, N, K, L, dtype, pdtype, w2.data(), w2.size(), nullptr);
     if (rc) { fprintf(stderr, "backward_params: %s\n", wtconv_last_error()); return 3; }
+    }
   }
   out.unpack(); dx.unpack();
   FILE* fo = fopen(argv[2], "wb");

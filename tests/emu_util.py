@@ -50,7 +50,7 @@ def half_roundtrip(values):
 
 
 def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, timeout=600, lds_limit=None,
-        mfma=None):
+        mfma=None, fused_bwd=False):
     """All arrays float32 numpy.  2-D: x (B,C,H,W); 1-D: x (B,C,N).  Returns dict of float32 arrays.
     `lds_limit` (bytes) lowers the LDS budget of the dispatch, so that small planes take the
     level-by-level kernels that real runs only use for planes beyond 160 KB."""
@@ -81,6 +81,9 @@ def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, 
         env.pop("WT_EMU_LDS_LIMIT", None)
         if lds_limit is not None:
             env["WT_EMU_LDS_LIMIT"] = str(int(lds_limit))
+        env.pop("WT_EMU_FUSED_BWD", None)
+        if fused_bwd:         # the backward pass as the single call wtconv*_backward instead of its two halves
+            env["WT_EMU_FUSED_BWD"] = "1"
         env.pop("WTCONV_MFMA", None)
         if mfma is not None:      # 0: vector-ALU kernels only; 1: matrix cores for bf16; 2: for bf16 and fp32
             env["WTCONV_MFMA"] = str(int(mfma))

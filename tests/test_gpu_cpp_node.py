@@ -141,3 +141,28 @@ def test_double_backward_is_refused(dev):
     (gx,) = torch.autograd.grad(out.sum(), x, create_graph=True)
     with pytest.raises(RuntimeError):
         gx.sum().backward()
+
+
+def test_gradient_penalty_is_refused_not_dropped(dev):
+    """A loss that mixes the output with a function of grad_x: the second-order term cannot be differentiated, and
+    both autograd paths must say so instead of treating it as a constant."""
+    params = _params(2, 4, 5, 1, True, torch.float32, dev)
+    for fn in _both(2, None, params, 5, 1):
+        x = torch.randn(2, 4, 10, 10, device=dev, requires_grad=True)
+        bw, bb, bs, ws, ss = params
+        out = fn(x, bw, bb, bs, ws, ss)
+        (gx,) = torch.autograd.grad(out.sum(), x, create_graph=True)
+        loss = out.sum() + gx.pow(2).sum()
+        with pytest.raises(RuntimeError):
+            loss.backward()
+
+
+def test_create_graph_without_second_order_use_still_works(dev):
+    """create_graph=True alone is harmless as long as nothing differentiates the gradients."""
+    params = _params(2, 4, 5, 1, True, torch.float32, dev)
+    cpp, py = _both(2, None, params, 5, 1)
+    bw, bb, bs, ws, ss = params
+    x = torch.randn(2, 4, 10, 10, device=dev, requires_grad=True)
+    (ga,) = torch.autograd.grad(cpp(x, bw, bb, bs, ws, ss).sum(), x, create_graph=True)
+    (gb,) = torch.autograd.grad(py(x, bw, bb, bs, ws, ss).sum(), x, create_graph=True)
+    assert torch.equal(ga.detach(), gb.detach())

@@ -618,7 +618,13 @@ def test_config2_full_size_fp32(hip_device):
 
 
 def test_config2_full_size_param_grads_vs_oracle(hip_device):
-    """All parameter gradients of config 2 at the full batch against the fp64 oracle."""
+    """All parameter gradients of config 2 at the full batch against the fp64 oracle.
+
+    The one exception to the stated fp32 bar (rtol 1e-5, atol 1e-4): the absolute floor of this test is
+    max(1e-4, 1e-6 * max|grad|) per tensor.  Each entry sums 128*56*56 = 401 408 products (|sum| up to a few
+    thousand), which float32 itself resolves only to ~1e-7 of its magnitude; the effective floor and the tensor's
+    largest entry are printed per tensor and named in the assertion message, next to the error of the CPU fp32
+    oracle against fp64."""
     W2, _ = _mods()
     ref, x, g = U.seeded_case("2d", 96, 5, 3, (128, 96, 56, 56))
     U.randomize_scales(ref)
@@ -634,15 +640,16 @@ def test_config2_full_size_param_grads_vs_oracle(hip_device):
         if n in ("wt_filter", "iwt_filter"):
             continue
         atol = max(U.FP32_ATOL, 1e-6 * want.abs().max().item())
+        wmax = want.abs().max().item()
         torch.testing.assert_close(gg[n].double(), want, rtol=U.FP32_RTOL, atol=atol,
-                                   msg=lambda m, n=n: f"{n}: {m}")
+                                   msg=lambda m, n=n, a=atol, w=wmax: f"{n} (max|want| = {w:.4g}, effective atol = {a:.3g}): {m}")
         e_hip = (gg[n].double() - want).abs().max().item()
         e_cpu = (wg32[n].double() - want).abs().max().item()
-        print(f"\n{n}: max|hip-fp64| = {e_hip:.3e}, max|cpu_fp32-fp64| = {e_cpu:.3e}, max|want| = {want.abs().max():.1f}")
+        print(f"\n{n}: max|hip-fp64| = {e_hip:.3e}, max|cpu_fp32-fp64| = {e_cpu:.3e}, max|want| = {wmax:.1f}, effective atol = {atol:.3g}")
 
 
 
-def _full_size_properties(kind, C, K, L, shape, hip_device, dtype, nsample=2):
+def _full_size_properties(kind, C, K, L, shape, hip_device, dtype, nsample=2, oracle_params=False):
     """Full-size run of one configuration: the first `nsample` batch items against the oracle
     (planes / rows are independent), the adjoint identity <f(x) - bias response, g> = <x, f^T g>
     over the whole batch (accumulated in float64 on the device) and additivity of the
@@ -685,12 +692,23 @@ def _full_size_properties(kind, C, K, L, shape, hip_device, dtype, nsample=2):
     for n in full:
         scale = full[n].abs().max().item()
         assert (full[n] - acc[n]).abs().max().item() <= 2e-5 * scale + 1e-4, n
+    if oracle_params:
+        # every parameter gradient of the whole batch against the oracle run on the whole batch (for bf16 tensors:
+        # fp32 maths on the bf16-rounded inputs), at the bar of the dtype
+        torch.set_num_threads(16)
+        _, _, wg = U.oracle_run(ref, x, g, torch.float32 if bf16 else torch.float64)
+        for n, want in wg.items():
+            if n in ("wt_filter", "iwt_filter"):
+                continue
+            check(full[n].float().cpu(), want.float(), f"{n} (full batch)")
 
 
 @pytest.mark.parametrize("name,C,L,H", [("2b", 96, 3, 56), ("3a", 192, 3, 28), ("3b", 384, 2, 14), ("3c", 768, 2, 7)])
 def test_full_size_bf16_configs(hip_device, name, C, L, H):
-    """The bf16 benchmark configurations (stage 1-4 shapes of WTConvNeXt-T) at their full sizes (batch 128)."""
-    _full_size_properties("2d", C, 5, L, (128, C, H, H), hip_device, torch.bfloat16)
+    """The bf16 benchmark configurations (stage 1-4 shapes of WTConvNeXt-T) at their full sizes (batch 128); the
+    parameter gradients of the whole batch are compared with the oracle as well (each entry sums up to 401 408
+    products of bf16-rounded operands)."""
+    _full_size_properties("2d", C, 5, L, (128, C, H, H), hip_device, torch.bfloat16, oracle_params=True)
 
 
 def test_config4_full_size_1d(hip_device):

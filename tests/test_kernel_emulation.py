@@ -272,3 +272,27 @@ def test_emulated_1d_row_resident_bf16():
     x, g = _bf16_round(x), _bf16_round(g)
     got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, 5, dtype=1)
     _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=1e-2, atol_scale=1e-2)
+
+
+@pytest.mark.parametrize("B,C,N,K,L,bias,dtype,pdtype", [
+    (3, 2, 1024, 5, 4, True, 0, 0),      # 32 full lanes; three batch items: chunks of uneven length, tickets of two channels
+    (1, 1, 2500, 5, 4, True, 0, 0),      # ragged last lane
+    (2, 2, 517, 5, 3, False, 0, 0),      # 16 samples per lane, odd length, element-wise HBM path, no bias
+    (1, 1, 700, 7, 3, True, 0, 0),       # K = 7
+    (1, 2, 800, 3, 5, True, 0, 0),       # five levels
+    (2, 1, 1000, 5, 4, True, 1, 1),      # bf16 rows and parameters
+    (1, 1, 17000, 5, 4, True, 0, 0),     # longer than the fused kernel takes: falls back to the two half passes
+])
+def test_emulated_1d_fused_backward(B, C, N, K, L, bias, dtype, pdtype):
+    """wtconv1d_backward as one call: grad_x and every parameter gradient from the fused row kernel (the last
+    workgroup of a channel runs the second stage)."""
+    x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, bias)
+    if dtype:
+        x, g = _bf16_round(x), _bf16_round(g)
+    if pdtype:
+        bw, bs = _bf16_round(bw), _bf16_round(bs)
+        bb = _bf16_round(bb) if bias else None
+        ws, ss = [_bf16_round(w) for w in ws], [_bf16_round(s) for s in ss]
+    got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K, dtype=dtype, pdtype=pdtype, fused_bwd=True)
+    tol = 1e-2 if dtype else 2e-5
+    _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=tol, atol_scale=tol)

@@ -20,6 +20,8 @@ def usable(x, *params):
         return False
     if torch.compiler.is_compiling():
         return False
+    if torch.is_autocast_enabled():      # autocast keeps LayerNorm outputs and the residual stream in fp32; the kernels return x.dtype
+        return False
     if not x.is_cuda or x.dtype not in _DT or x.dim() != 4 or x.shape[1] % 2 or not x.is_contiguous():
         return False
     pd = None
@@ -30,6 +32,14 @@ def usable(x, *params):
             return False
         pd = p.dtype
     return True
+
+
+def usable_nhwc(y, shortcut):
+    """Whether block_residual takes the MLP output `y` (B, H, W, C) for this shortcut: nothing recorded for autograd
+    on it, same dtype and device as the shortcut."""
+    if torch.is_grad_enabled() and y.requires_grad:
+        return False
+    return y.dtype == shortcut.dtype and y.device == shortcut.device and y.dim() == 4
 
 
 def _stream():

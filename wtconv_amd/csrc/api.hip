@@ -469,17 +469,20 @@ static int run_wgrad1d_k(int K, int L, const void* x, const void* g, float* part
 }
 
 // ---- row-resident 1-D kernels ----------------------------------------------------------
-// Rows of 16 to 512 lanes' worth of samples run on the register-resident kernels; shorter or
-// longer rows, K = 1 and (K, L) pairs whose lane would hold more than 32 samples use the tiled ones.
-static bool row1d_lanes(int N, int K, int L, int* nl, int* block) {
-  if (K < 3 || K > 7 || L < 1 || L > kMaxLevels) return false;
-  const int S = row1d_samples(K, L);
-  if (S > kRow1dMaxSamples) return false;
-  const int n = (N + S - 1) / S;
-  if (n < 16 || n > kRow1dMaxLanes) return false;
-  *nl = n;
-  *block = (n + 63) / 64 * 64;
-  return true;
+// Rows of 16 to `max_lanes` lanes' worth of samples run on the register-resident kernels, with 16 samples per lane
+// where the row fits the workgroup that way and 32 otherwise; shorter or longer rows and K = 1 use the tiled ones.
+struct Row1DShape { int S, nl, block; };
+
+static bool row1d_shape(int N, int K, int L, int max_lanes, Row1DShape* sh) {
+  if (K < 3 || K > 7 || L < 1 || L > kMaxLevels || N <= 0) return false;
+  for (int S : {16, 32}) {
+    if (!row1d_built(K, L, S)) continue;
+    const int n = (N + S - 1) / S;
+    if (n < 16 || n > max_lanes) continue;
+    sh->S = S; sh->nl = n; sh->block = (n + 63) / 64 * 64;
+    return true;
+  }
+  return false;
 }
 
 static Row1D make_row1d(int C, int N, int nl, size_t esz, const void* p0, const void* p1) {
@@ -490,14 +493,12 @@ static Row1D make_row1d(int C, int N, int nl, size_t esz, const void* p0, const 
   return r;
 }
 
-// Rows per workgroup of the row-resident weight-gradient kernel: enough chunks to fill 256 CUs
-// at 8 waves each (a constant, so that workspace sizes do not depend on the device queried).
-static void row1d_chunks(int B, int C, int K, int L, int block, int* per_chunk, int* nchunk) {
-  const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
-  int per_cu = static_cast<int>(kLdsLimitBytes / lds);
-  if (per_cu > 512 / block) per_cu = 512 / block;
+// Batch chunks of a row-resident kernel: C * nchunk workgroups that all run at once (one round: a second, partly
+// filled round costs as much as a full one), `per_cu` of them per CU on 256 CUs -- constants, so that workspace
+// sizes do not depend on the device queried.
+static void row1d_chunks(int B, int C, int per_cu, int* per_chunk, int* nchunk) {
   if (per_cu < 1) per_cu = 1;
-  int want = (256 * per_cu + C - 1) / C;
+  int want = 256 * per_cu / C;
   if (want < 1) want = 1;
   if (want > B) want = B;
   const int pc = (B + want - 1) / want;
@@ -505,31 +506,60 @@ static void row1d_chunks(int B, int C, int K, int L, int block, int* per_chunk, 
   *nchunk = (B + pc - 1) / pc;
 }
 
-template <typename T, int K, int L>
-static int run_row1d(const void* x, void* out, const float* fw, const float* fb, const Row1D& pl, int B, int block,
-                     hipStream_t stream) {
-  if constexpr (row1d_built(K, L)) {
-    auto kern = wt1d_row_kernel<T, K, L>;
-    const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
+// Workgroups per CU the kernels with two slot regions (parameter gradients, fused backward) are planned for: what
+// LDS allows, at most two waves per SIMD (they need up to 256 registers).
+static int row1d_two_region_per_cu(int K, int L, const Row1DShape& sh) {
+  const size_t lds = 2 * row1d_region(K, L, sh.S, sh.block) * sizeof(float);
+  int per_cu = static_cast<int>(kLdsLimitBytes / lds);
+  if (per_cu > 512 / sh.block) per_cu = 512 / sh.block;
+  return per_cu < 1 ? 1 : per_cu;
+}
+
+template <typename T, int K, int L, int S>
+static int run_row1d(const void* x, void* out, const wtconv_params* params, int pdtype, int flip, const Row1D& pl,
+                     int B, int block, hipStream_t stream) {
+  if constexpr (row1d_built(K, L, S)) {
+    auto kern = wt1d_row_kernel<T, K, L, S>;
+    const size_t lds = row1d_region(K, L, S, block) * sizeof(float);
     if (int e = allow_lds(kern, lds)) return e;
-    const long long nrows = static_cast<long long>(B) * pl.C;
-    if (nrows > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "batch*channels = %lld is too large", nrows);
-    long long grid = static_cast<long long>(compute_units()) * resident_per_cu(kern, block, lds);
-    if (grid > nrows) grid = nrows;
-    WT_LAUNCH(kern, dim3(static_cast<unsigned>(grid)), dim3(block), lds, stream, static_cast<const T*>(x),
-              static_cast<T*>(out), fw, fb, pl, static_cast<int>(nrows));
+    int per_chunk, nchunk;
+    row1d_chunks(B, pl.C, resident_per_cu(kern, block, lds), &per_chunk, &nchunk);   // (no workspace depends on this)
+    if (nchunk > 65535) return fail(WTCONV_E_UNSUPPORTED, "too many batch chunks (%d)", nchunk);
+    WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(block), lds, stream, static_cast<const T*>(x), static_cast<T*>(out),
+              to_table(params, L), pdtype, flip, pl, B, per_chunk);
     return check_launch("wt1d_row_kernel");
   } else {
     return fail(WTCONV_E_UNSUPPORTED, "row-resident 1-D kernel not built for kernel_size %d, %d levels", K, L);
   }
 }
 
-template <typename T, int K, int L>
+// The fused backward kernel: grad_x, the chunks' partial sums and (by the last workgroup of each channel) the
+// parameter gradients.  `tickets`: C words, cleared by a launch of their own right before.
+template <typename T, int K, int L, int S>
+static int run_row1d_bwd(const void* x, const void* g, void* gx, float* partial, unsigned* tickets,
+                         const wtconv_params* params, int pdtype, const GradTable& gt, const Row1D& pl, int B,
+                         int block, int per_chunk, int nchunk, hipStream_t stream) {
+  if constexpr (row1d_bwd_built(K, L, S)) {
+    auto kern = wt1d_row_bwd_kernel<T, K, L, S>;
+    const size_t lds = 2 * row1d_region(K, L, S, block) * sizeof(float);
+    if (int e = allow_lds(kern, lds)) return e;
+    WT_LAUNCH(zero_tickets_kernel, dim3((pl.C + 255) / 256), dim3(256), 0, stream, tickets, pl.C);
+    if (int e = check_launch("zero_tickets_kernel")) return e;
+    WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(block), lds, stream, static_cast<const T*>(x),
+              static_cast<const T*>(g), static_cast<T*>(gx), partial, tickets, to_table(params, L), pdtype, gt, pl, B,
+              per_chunk, nchunk);
+    return check_launch("wt1d_row_bwd_kernel");
+  } else {
+    return fail(WTCONV_E_UNSUPPORTED, "row-resident 1-D kernel not built for kernel_size %d, %d levels", K, L);
+  }
+}
+
+template <typename T, int K, int L, int S>
 static int run_row1d_wgrad(const void* x, const void* g, float* partial, const Row1D& pl, int B, int block,
                            int per_chunk, int nchunk, hipStream_t stream) {
-  if constexpr (row1d_built(K, L)) {
-    auto kern = wt1d_row_wgrad_kernel<T, K, L>;
-    const size_t lds = static_cast<size_t>(2) * block * row1d_slot(K, L) * sizeof(float);
+  if constexpr (row1d_built(K, L, S)) {
+    auto kern = wt1d_row_wgrad_kernel<T, K, L, S>;
+    const size_t lds = 2 * row1d_region(K, L, S, block) * sizeof(float);
     if (int e = allow_lds(kern, lds)) return e;
     WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(block), lds, stream, static_cast<const T*>(x),
               static_cast<const T*>(g), partial, pl, B, per_chunk);
@@ -539,13 +569,15 @@ static int run_row1d_wgrad(const void* x, const void* g, float* partial, const R
   }
 }
 
+#define WT_ROW1D_SWITCH_S(T, K, L, CALL)                              \
+  return S == 16 ? CALL(T, K, L, 16) : CALL(T, K, L, 32);
 #define WT_ROW1D_SWITCH_L(T, K, CALL)                                 \
   switch (L) {                                                        \
-    case 1: return CALL(T, K, 1);                                     \
-    case 2: return CALL(T, K, 2);                                     \
-    case 3: return CALL(T, K, 3);                                     \
-    case 4: return CALL(T, K, 4);                                     \
-    case 5: return CALL(T, K, 5);                                     \
+    case 1: WT_ROW1D_SWITCH_S(T, K, 1, CALL)                          \
+    case 2: WT_ROW1D_SWITCH_S(T, K, 2, CALL)                          \
+    case 3: WT_ROW1D_SWITCH_S(T, K, 3, CALL)                          \
+    case 4: WT_ROW1D_SWITCH_S(T, K, 4, CALL)                          \
+    case 5: WT_ROW1D_SWITCH_S(T, K, 5, CALL)                          \
   }                                                                   \
   break;
 #define WT_ROW1D_SWITCH(T, CALL)                                      \
@@ -556,18 +588,31 @@ static int run_row1d_wgrad(const void* x, const void* g, float* partial, const R
   }
 
 template <typename T>
-static int run_row1d_kl(int K, int L, const void* x, void* out, const float* fw, const float* fb, const Row1D& pl,
-                        int B, int block, hipStream_t stream) {
-#define WT_CALL(T_, K_, L_) run_row1d<T_, K_, L_>(x, out, fw, fb, pl, B, block, stream)
+static int run_row1d_kl(int K, int L, int S, const void* x, void* out, const wtconv_params* params, int pdtype,
+                        int flip, const Row1D& pl, int B, int block, hipStream_t stream) {
+#define WT_CALL(T_, K_, L_, S_) run_row1d<T_, K_, L_, S_>(x, out, params, pdtype, flip, pl, B, block, stream)
   WT_ROW1D_SWITCH(T, WT_CALL)
 #undef WT_CALL
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d / %d levels not built", K, L);
 }
 
 template <typename T>
-static int run_row1d_wgrad_kl(int K, int L, const void* x, const void* g, float* partial, const Row1D& pl, int B,
-                              int block, int per_chunk, int nchunk, hipStream_t stream) {
-#define WT_CALL(T_, K_, L_) run_row1d_wgrad<T_, K_, L_>(x, g, partial, pl, B, block, per_chunk, nchunk, stream)
+static int run_row1d_bwd_kl(int K, int L, int S, const void* x, const void* g, void* gx, float* partial,
+                            unsigned* tickets, const wtconv_params* params, int pdtype, const GradTable& gt,
+                            const Row1D& pl, int B, int block, int per_chunk, int nchunk, hipStream_t stream) {
+#define WT_CALL(T_, K_, L_, S_)                                                                                 \
+  run_row1d_bwd<T_, K_, L_, S_>(x, g, gx, partial, tickets, params, pdtype, gt, pl, B, block, per_chunk, nchunk, \
+                                stream)
+  WT_ROW1D_SWITCH(T, WT_CALL)
+#undef WT_CALL
+  return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d / %d levels not built", K, L);
+}
+
+template <typename T>
+static int run_row1d_wgrad_kl(int K, int L, int S, const void* x, const void* g, float* partial, const Row1D& pl,
+                              int B, int block, int per_chunk, int nchunk, hipStream_t stream) {
+#define WT_CALL(T_, K_, L_, S_) \
+  run_row1d_wgrad<T_, K_, L_, S_>(x, g, partial, pl, B, block, per_chunk, nchunk, stream)
   WT_ROW1D_SWITCH(T, WT_CALL)
 #undef WT_CALL
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d / %d levels not built", K, L);
@@ -582,20 +627,20 @@ static int tile1d_pass(const char* fn, const void* x, void* out, const wtconv_pa
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(out) % esz))
     return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
-  int nl = 0, block = 0;
-  const bool row_resident = row1d_lanes(N, K, L, &nl, &block);
+  Row1DShape sh = {};
+  const bool row_resident = row1d_shape(N, K, L, kRow1dMaxLanes, &sh);
   const Plan1D pl = make_plan1d(C, N, K, L, false, esz, x, out, nullptr);
   const size_t need = wtconv1d_workspace_bytes(B, C, N, K, L, flip ? WTCONV_PASS_BACKWARD_INPUT : WTCONV_PASS_FORWARD);
   if (ws == nullptr || ws_bytes < need)
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, ws_bytes);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (row_resident) {      // (these kernels fold their channel's parameters themselves: no fold launch, no table)
+    const Row1D rp = make_row1d(C, N, sh.nl, esz, x, out);
+    return WT_BY_DTYPE(dtype, run_row1d_kl<T_>(K, L, sh.S, x, out, params, pdtype, flip, rp, B, sh.block, stream));
+  }
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 2 * L) * K;
   if (int e = launch_fold(params, pdtype, fw, fb, C, 2, L, K, flip, flip ? 0 : 1, stream)) return e;
-  if (row_resident) {
-    const Row1D rp = make_row1d(C, N, nl, esz, x, out);
-    return WT_BY_DTYPE(dtype, run_row1d_kl<T_>(K, L, x, out, fw, fb, rp, B, block, stream));
-  }
   return WT_BY_DTYPE(dtype, run_tile1d_k<T_>(K, x, out, fw, fb, pl, B, stream));
 }
 
@@ -794,12 +839,14 @@ size_t wtconv1d_workspace_bytes(int B, int C, int N, int K, int levels, int pass
   size_t floats;
   if (pass == WTCONV_PASS_BACKWARD_PARAMS) {
     const Plan1D pl = make_plan1d(C, N, K, levels, true, 4, nullptr, nullptr, nullptr);
-    int per_chunk, nchunk, nl = 0, block = 0;
-    if (row1d_lanes(N, K, levels, &nl, &block))
-      row1d_chunks(B, C, K, levels, block, &per_chunk, &nchunk);
+    int per_chunk, nchunk;
+    Row1DShape sh = {};
+    if (row1d_shape(N, K, levels, kRow1dMaxLanes, &sh))
+      row1d_chunks(B, C, row1d_two_region_per_cu(K, levels, sh), &per_chunk, &nchunk);
     else
       wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
-    floats = static_cast<size_t>(nchunk) * C * ((1 + 2 * levels) * K + 1);
+    // partial sums, then one ticket word per channel (fused backward kernel)
+    floats = round_up64(static_cast<size_t>(nchunk) * C * ((1 + 2 * levels) * K + 1)) + static_cast<size_t>(C);
   } else {
     floats = fold_floats(C, 2, levels, K);
   }
@@ -843,18 +890,20 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   if (workspace == nullptr || workspace_bytes < need)
     return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  int per_chunk, nchunk, nl = 0, block = 0;
-  const bool row_resident = row1d_lanes(N, K, L, &nl, &block);
+  int per_chunk, nchunk;
+  Row1DShape sh = {};
+  const bool row_resident = row1d_shape(N, K, L, kRow1dMaxLanes, &sh);
   if (row_resident)
-    row1d_chunks(B, C, K, L, block, &per_chunk, &nchunk);
+    row1d_chunks(B, C, row1d_two_region_per_cu(K, L, sh), &per_chunk, &nchunk);
   else
     wgrad_chunks1d(B, C, pl.ntiles, &per_chunk, &nchunk);
   if (nchunk > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
   float* partial = static_cast<float*>(workspace);
   int e;
   if (row_resident) {
-    const Row1D rp = make_row1d(C, N, nl, esz, x, grad_out);
-    e = WT_BY_DTYPE(dtype, run_row1d_wgrad_kl<T_>(K, L, x, grad_out, partial, rp, B, block, per_chunk, nchunk, stream));
+    const Row1D rp = make_row1d(C, N, sh.nl, esz, x, grad_out);
+    e = WT_BY_DTYPE(dtype, run_row1d_wgrad_kl<T_>(K, L, sh.S, x, grad_out, partial, rp, B, sh.block, per_chunk, nchunk,
+                                                  stream));
   } else {
     e = WT_BY_DTYPE(dtype, run_wgrad1d_k<T_>(K, L, x, grad_out, partial, pl, B, per_chunk, nchunk, stream));
   }
@@ -870,9 +919,60 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   return check_launch("wgrad_finish_kernel");
 }
 
+static int check_grad_table(const char* fn, const wtconv_params* params, const wtconv_param_grads* grads, int L) {
+  if (grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
+      (params->base_bias != nullptr && grads->base_bias == nullptr))
+    return fail(WTCONV_E_ARG, "%s: null gradient pointer", fn);
+  for (int l = 0; l < L; ++l)
+    if (grads->wt_weight[l] == nullptr || grads->wt_scale[l] == nullptr)
+      return fail(WTCONV_E_ARG, "%s: null gradient pointer at level %d", fn, l);
+  return 0;
+}
+
+static GradTable to_grad_table(const wtconv_param_grads* grads, int L) {
+  GradTable gt = {};
+  gt.base_weight = grads->base_weight;
+  gt.base_bias = grads->base_bias;
+  gt.base_scale = grads->base_scale;
+  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
+  return gt;
+}
+
 int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
                       const wtconv_param_grads* grads, int B, int C, int N, int K, int levels, int dtype,
                       int param_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* fn = "wtconv1d_backward";
+  // rows that the register-resident kernels take run the whole backward pass as one kernel -- with the lanes, chunks
+  // and workspace layout of the separate parameter-gradient pass, so the two share wtconv1d_workspace_bytes
+  Row1DShape sh = {};
+  if (K >= 1 && levels >= 1 && levels <= kMaxLevels && row1d_shape(N, K, levels, kRow1dMaxLanes, &sh) &&
+      sh.block <= kRow1dBwdMaxLanes && row1d_bwd_built(K, levels, sh.S)) {
+    const int L = levels;
+    if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
+    if (x == nullptr || grad_out == nullptr || grad_x == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+    if (int e = check_grad_table(fn, params, grads, L)) return e;
+    const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+    if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(grad_out) % esz) ||
+        (reinterpret_cast<uintptr_t>(grad_x) % esz))
+      return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned to its element size", fn);
+    const size_t need = wtconv1d_workspace_bytes(B, C, N, K, L, WTCONV_PASS_BACKWARD);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+    if (reinterpret_cast<uintptr_t>(workspace) % 4)
+      return fail(WTCONV_E_ARG, "%s: workspace not aligned", fn);
+    int per_chunk, nchunk;
+    row1d_chunks(B, C, row1d_two_region_per_cu(K, L, sh), &per_chunk, &nchunk);
+    if (nchunk > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
+    float* partial = static_cast<float*>(workspace);
+    unsigned* tickets = reinterpret_cast<unsigned*>(partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 2 * L) * K + 1)));
+    Row1D rp = make_row1d(C, N, sh.nl, esz, x, grad_out);
+    rp.vec_ok = rp.vec_ok && (reinterpret_cast<uintptr_t>(grad_x) & 15u) == 0;
+    const GradTable gt = to_grad_table(grads, L);
+    return WT_BY_DTYPE(dtype, run_row1d_bwd_kl<T_>(K, L, sh.S, x, grad_out, grad_x, partial, tickets, params, param_dtype,
+                                                    gt, rp, B, sh.block, per_chunk, nchunk,
+                                                    static_cast<hipStream_t>(stream)));
+  }
   if (int e = wtconv1d_backward_input(grad_out, grad_x, params, B, C, N, K, levels, dtype, param_dtype, workspace,
                                       workspace_bytes, stream))
     return e;

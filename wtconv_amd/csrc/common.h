@@ -214,6 +214,80 @@ struct GradTable {
   float* wt_scale[kMaxLevels];
 };
 
+// Value of lane `src` (a constant) of the calling wavefront, as a wave-uniform value (v_readlane_b32: the result lives
+// in an SGPR, so an FMA takes it as its scalar operand).  The host emulation has no lanes to read from: there every
+// thread holds the whole table and indexes it itself (see LaneTable).
+#ifndef WT_EMULATE
+__device__ __forceinline__ float lane_bcast(float v, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+#endif
+
+// N wave-uniform floats kept one per lane: entry i in lane i % 64 of word i / 64 of every wavefront (N / 64 vector
+// registers instead of N; reading entry i costs one v_readlane).  This is how the vector-ALU kernels hold the
+// folded parameters of their channel when they fold them themselves.
+template <int N>
+struct LaneTable {
+#ifdef WT_EMULATE
+  float v[N];
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+  template <typename F> __device__ __forceinline__ void fill(F&& f) {
+    for (int i = 0; i < N; ++i) v[i] = f(i);
+  }
+#else
+  static constexpr int kWords = (N + kWave - 1) / kWave;
+  float v[kWords];
+  // `i` must be a compile-time constant after unrolling (v_readlane takes the lane as an immediate or an SGPR)
+  __device__ __forceinline__ float get(int i) const { return lane_bcast(v[i / kWave], i % kWave); }
+  // f(i) is evaluated by the lane that keeps entry i
+  template <typename F> __device__ __forceinline__ void fill(F&& f) {
+    const int lane = static_cast<int>(threadIdx.x) & (kWave - 1);
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) {
+      const int i = lane + j * kWave;
+      v[j] = i < N ? f(i) : 0.f;
+    }
+  }
+#endif
+};
+
+// Hand-over between the workgroups of one launch.  What a workgroup leaves for another one to read (its record of
+// partial sums) is stored with store_shared_f32 and read with load_shared_f32: device-scope accesses that go through
+// to / come from the memory all compute units see, whichever L2 the two workgroups sit behind.  No cache is written
+// back or invalidated as a whole (a device-scope fence would do that once per workgroup, and every one of them would
+// have to go through everything the launch has written so far).
+#ifdef WT_EMULATE
+__device__ __forceinline__ void store_shared_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ float load_shared_f32(const float* p) { return *p; }
+#else
+__device__ __forceinline__ void store_shared_f32(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared_f32(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+#endif
+
+// Every thread calls this after its store_shared_f32 stores: they are waited for, one ticket is drawn, and the call
+// returns true in the workgroup that drew the last of `total` (the same value in all its threads), which may then
+// read with load_shared_f32 what every other workgroup stored before its own call.  `flag` = one word of LDS.  The
+// ticket word must be zero when the launch starts; the last workgroup leaves it zero again.
+__device__ __forceinline__ bool workgroup_is_last(unsigned* __restrict__ ticket, unsigned total, unsigned* flag) {
+#ifdef WT_EMULATE
+  __syncthreads();
+  if (threadIdx.x == 0) { *flag = (*ticket == total - 1) ? 1u : 0u; *ticket += 1u; }   // (workgroups run one after the other)
+  __syncthreads();
+  return *flag != 0u;
+#else
+  __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this thread's stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0)
+    *flag = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total - 1 ? 1u : 0u;
+  __syncthreads();
+  return *flag != 0u;
+#endif
+}
+
 // Orders the computation of v[] before the next WT_CHUNK_FENCE (the fence alone only
 // orders memory operations; arithmetic would otherwise be sunk below it and every row read
 // of a work item would stay live at once).  Emits no instruction.

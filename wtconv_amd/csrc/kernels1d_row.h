@@ -14,23 +14,31 @@
 // Maths as in kernels1d.h (reference wtconv/wtconv1d.py:38-82, wtconv/util/wavelet.py:6-20,
 // 46-59).  Samples past the end of the row are staged as zeros, which gives the 'same'
 // padding of every level and the zero padding of odd lengths at once.
+//
+// A workgroup works on rows of ONE channel (grid = channels x batch chunks), and folds that
+// channel's parameters itself when it starts (gamma * w, taps reversed for the input gradient):
+// one entry per lane, read back as wave-uniform values -- no fold launch, no folded table in
+// HBM.  The backward pass is one kernel: the row of x and the row of grad_out are read once and
+// give grad_x and the running sums of the parameter gradients; the workgroup that finishes a
+// channel last (a ticket per channel) sums the chunks' partial sums in chunk order and writes
+// the channel's parameter gradients.
 #pragma once
 
 #include "common.h"
 #include "kernels1d.h"
+#include "kernels2d.h"      // wgrad_finish_channel
 
 namespace wt {
 
-// Samples per lane: a multiple of 2^L (the pyramid of a lane is local) and of 8 (16-byte
-// vectors of either dtype).  32 from four levels on (measured faster than 16 at L = 4: fewer
-// edge exchanges per sample), 16 below.
-constexpr int row1d_samples(int K, int L) {
-  (void)K;
-  return L >= 4 ? 32 : 16;
-}
+// Samples per lane S: a multiple of 2^L (the pyramid of a lane is local) and of 8 (16-byte vectors of either
+// dtype): 16 or 32.  16 wherever the row fits the workgroup with it (twice the lanes per row, half the registers
+// per lane: more waves in flight, which is what these latency-bound kernels need), 32 for longer rows and for
+// five levels.
 constexpr int kRow1dMaxSamples = 32;
 constexpr int kRow1dMaxLanes = 512;      // threads per workgroup
-constexpr bool row1d_built(int K, int L) { return K >= 3 && row1d_samples(K, L) <= kRow1dMaxSamples; }
+constexpr bool row1d_built(int K, int L, int S) {
+  return K >= 3 && (S == 16 || S == 32) && S % (1 << L) == 0;
+}
 
 // Edge entries a lane publishes of an array of n entries: the first and last R, or all of
 // them when there are fewer than 2R.
@@ -46,13 +54,25 @@ constexpr int row1d_edge_off(int K, int S, int a) {
 
 // Floats of LDS per lane: the lane's S samples (plus a pad that makes the stride an odd
 // number of 16-byte units) or its published edges, whichever is larger.
-constexpr int row1d_slot(int K, int L) {
-  const int S = row1d_samples(K, L);
+constexpr int row1d_slot(int K, int L, int S) {
   const int halo = row1d_edge_off(K, S, 1 + 2 * L);
   int f = S + 4 > halo ? S + 4 : halo;
   f = (f + 3) / 4 * 4;
   if ((f / 4) % 2 == 0) f += 4;
   return f;
+}
+
+// Zero slots on either side of a region's `block` lane slots: a lane reads the edges of up to ceil(R / n) lanes
+// away (n = entries per lane at the coarsest level), and beyond either end of the row those reads land here --
+// no condition, no branch around the read, every edge at a constant offset from the lane's own slot.
+constexpr int row1d_guard(int K, int L, int S) {
+  const int nmin = S >> L;
+  const int R = K / 2;
+  return nmin < 1 ? R : (R + nmin - 1) / nmin;
+}
+// Floats of one region (guards included) for a workgroup of `block` lanes.
+constexpr size_t row1d_region(int K, int L, int S, int block) {
+  return static_cast<size_t>(block + 2 * row1d_guard(K, L, S)) * row1d_slot(K, L, S);
 }
 
 struct Row1D {
@@ -215,6 +235,18 @@ __device__ __forceinline__ void row1d_unstage(T* __restrict__ row, const float* 
   }
 }
 
+// Zeroes the guard slots of the `nregion` regions that start at `lds` (once per workgroup: nothing else writes them).
+template <int K, int L, int S>
+__device__ __forceinline__ void row1d_zero_guards(float* __restrict__ lds, int nregion, int tid, int nth) {
+  constexpr int SLOT = row1d_slot(K, L, S), G = row1d_guard(K, L, S);
+  const int rfl = (nth + 2 * G) * SLOT;
+  for (int r = 0; r < nregion; ++r)
+    for (int i = tid; i < 2 * G * SLOT; i += nth) {
+      const int off = i < G * SLOT ? i : rfl - 2 * G * SLOT + i;
+      lds[r * rfl + off] = 0.f;
+    }
+}
+
 template <int S>
 __device__ __forceinline__ void row1d_read_slot(const float* __restrict__ slot, float (&v)[S]) {
 #pragma unroll
@@ -283,12 +315,15 @@ __device__ __forceinline__ void row1d_publish_levels(float* __restrict__ slot, c
 
 // ext = [R entries to the left | the lane's n entries | R entries to the right] of array A;
 // the neighbours' entries come from the slots of the lanes that own them (one or, on coarse
-// levels with n < R, several lanes away); beyond either end of the workgroup they are zero.
+// levels with n < R, several lanes away); beyond either end of the workgroup those are the
+// region's zero guard slots.
 template <int K, int S, int SLOT, int A, int NA>
 __device__ __forceinline__ void row1d_extend(const float* __restrict__ region, int tid, int nth,
                                              const float (&arr)[NA],
                                              float (&ext)[row1d_len(S, A) + 2 * (K / 2)]) {
+  (void)nth;
   constexpr int R = K / 2, n = row1d_len(S, A), OFF = row1d_edge_off(K, S, A);
+  const float* own = region + tid * SLOT;
 #pragma unroll
   for (int d = 0; d < R; ++d) {
     {                                              // entry -R + d
@@ -296,23 +331,88 @@ __device__ __forceinline__ void row1d_extend(const float* __restrict__ region, i
       const int o = (e + n - 1) / n;               // lanes to the left
       const int loc = o * n - e;                   // its index in that lane's array
       const int pos = n < 2 * R ? loc : R + loc - (n - R);
-      ext[d] = tid - o >= 0 ? region[(tid - o) * SLOT + OFF + pos] : 0.f;
+      ext[d] = own[-o * SLOT + OFF + pos];
     }
     {                                              // entry n + d
       const int o = (n + d) / n;
       const int loc = (n + d) - o * n;
-      ext[R + n + d] = tid + o < nth ? region[(tid + o) * SLOT + OFF + loc] : 0.f;
+      ext[R + n + d] = own[o * SLOT + OFF + loc];
     }
   }
 #pragma unroll
   for (int q = 0; q < n; ++q) ext[R + q] = arr[q];
 }
 
-template <int K, int n>
-__device__ __forceinline__ void row1d_conv(const float (&ext)[n + K - 1], wt_uniform_ptr w, float (&y)[n]) {
+// The edges of every array of a lane's neighbours, fetched in one go (all the LDS reads of a row are in flight together
+// and waited for once): v[A][0..R) the R entries to the left of the lane's array A, v[A][R..2R) the R to its right.
+template <int K, int L>
+struct RowEdges { float v[1 + 2 * L][2 * (K / 2) > 0 ? 2 * (K / 2) : 1]; };
+
+template <int K, int S, int SLOT, int L, int A>
+__device__ __forceinline__ void row1d_load_edges_from(const float* __restrict__ own, RowEdges<K, L>& ed) {
+  if constexpr (A <= 2 * L) {
+    constexpr int R = K / 2, n = row1d_len(S, A), OFF = row1d_edge_off(K, S, A);
+#pragma unroll
+    for (int d = 0; d < R; ++d) {
+      {
+        const int e = R - d, o = (e + n - 1) / n, loc = o * n - e;
+        const int pos = n < 2 * R ? loc : R + loc - (n - R);
+        ed.v[A][d] = own[-o * SLOT + OFF + pos];
+      }
+      {
+        const int o = (n + d) / n, loc = (n + d) - o * n;
+        ed.v[A][R + d] = own[o * SLOT + OFF + loc];
+      }
+    }
+    row1d_load_edges_from<K, S, SLOT, L, A + 1>(own, ed);
+  }
+}
+
+template <int K, int S, int SLOT, int L>
+__device__ __forceinline__ void row1d_load_edges(const float* __restrict__ region, int tid, RowEdges<K, L>& ed) {
+  row1d_load_edges_from<K, S, SLOT, L, 0>(region + tid * SLOT, ed);
+}
+
+// ext of array A from edges fetched earlier
+template <int K, int S, int L, int A, int NA>
+__device__ __forceinline__ void row1d_extend_with(const RowEdges<K, L>& ed, const float (&arr)[NA],
+                                                  float (&ext)[row1d_len(S, A) + 2 * (K / 2)]) {
+  constexpr int R = K / 2, n = row1d_len(S, A);
+#pragma unroll
+  for (int d = 0; d < R; ++d) { ext[d] = ed.v[A][d]; ext[R + n + d] = ed.v[A][R + d]; }
+#pragma unroll
+  for (int q = 0; q < n; ++q) ext[R + q] = arr[q];
+}
+
+// Folded parameters of one channel: entry f * K + k = gamma[f] * w[f][k] (k reversed when flip != 0), f = 0 base
+// conv, f = 1 + 2 (l - 1) + s level l sub-band s.  The same products as fold_params_kernel forms.
+template <int K, int L>
+using RowWeights = LaneTable<(1 + 2 * L) * K>;
+
+template <int K, int L>
+__device__ __forceinline__ void row1d_fold(const ParamTable& p, int pdtype, int c, int flip, RowWeights<K, L>& tab) {
+  tab.fill([&](int i) {
+    const int f = i / K, t = i - f * K;
+    const int ts = flip ? K - 1 - t : t;
+    float v = 0.f;
+    if (f == 0) v = load_param(p.base_weight, pdtype, c * K + ts) * load_param(p.base_scale, pdtype, c);
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+      if (f >= 1 + 2 * l && f < 3 + 2 * l) {
+        const int ch = c * 2 + (f - 1 - 2 * l);
+        v = load_param(p.wt_weight[l], pdtype, ch * K + ts) * load_param(p.wt_scale[l], pdtype, ch);
+      }
+    }
+    return v;
+  });
+}
+
+// y += (filter F of the channel) (*) ext
+template <int K, int L, int F, int n>
+__device__ __forceinline__ void row1d_conv(const float (&ext)[n + K - 1], const RowWeights<K, L>& w, float (&y)[n]) {
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    const float wv = w[k];
+    const float wv = w.get(F * K + k);
 #pragma unroll
     for (int q = 0; q < n; ++q) y[q] = fmaf(wv, ext[q + k], y[q]);
   }
@@ -322,7 +422,7 @@ __device__ __forceinline__ void row1d_conv(const float (&ext)[n + K - 1], wt_uni
 // entry when l < L; the level-1 reconstruction is added into `out`.
 template <int K, int S, int SLOT, int L, int l>
 __device__ __forceinline__ void row1d_synth(const RowPyramid<S, L>& py, const float* __restrict__ region, int tid,
-                                            int nth, wt_uniform_ptr fwc, float (&zc)[S / 2], float (&out)[S]) {
+                                            int nth, const RowWeights<K, L>& fwc, float (&zc)[S / 2], float (&out)[S]) {
   if constexpr (l >= 1) {
     constexpr int R = K / 2;
     constexpr int n = S >> l;
@@ -332,12 +432,12 @@ __device__ __forceinline__ void row1d_synth(const RowPyramid<S, L>& py, const fl
     {
       float ext[n + 2 * R];
       row1d_extend<K, S, SLOT, 1 + 2 * (l - 1)>(region, tid, nth, py.lo[l - 1], ext);
-      row1d_conv<K, n>(ext, fwc + (1 + 2 * (l - 1)) * K, ylo);
+      row1d_conv<K, L, 1 + 2 * (l - 1), n>(ext, fwc, ylo);
     }
     {
       float ext[n + 2 * R];
       row1d_extend<K, S, SLOT, 2 + 2 * (l - 1)>(region, tid, nth, py.hi[l - 1], ext);
-      row1d_conv<K, n>(ext, fwc + (2 + 2 * (l - 1)) * K, yhi);
+      row1d_conv<K, L, 2 + 2 * (l - 1), n>(ext, fwc, yhi);
     }
     if constexpr (l > 1) {
 #pragma unroll
@@ -353,87 +453,6 @@ __device__ __forceinline__ void row1d_synth(const RowPyramid<S, L>& py, const fl
       }
     }
     row1d_synth<K, S, SLOT, L, l - 1>(py, region, tid, nth, fwc, zc, out);
-  }
-}
-
-// Forward / input-gradient kernel.  Persistent: grid = min(rows, resident workgroups), block =
-// lanes (multiple of 64, >= ceil(N / S)), dynamic LDS = 2 * block * SLOT floats: two slot
-// regions that alternate between rows.  The next row of the workgroup is fetched into
-// registers while the current one is computed and committed to the other region before the
-// current outputs are stored, so that loads never wait behind stores; three barriers per row.
-template <typename T, int K, int L>
-__global__ __launch_bounds__(kRow1dMaxLanes) void wt1d_row_kernel(const T* __restrict__ x, T* __restrict__ out,
-                                                                   const float* __restrict__ fw,
-                                                                   const float* __restrict__ fb, Row1D pl,
-                                                                   int nrows) {
-  WT_SHARED_FLOATS(lds);
-  constexpr int R = K / 2;
-  constexpr int S = row1d_samples(K, L);
-  constexpr int SLOT = row1d_slot(K, L);
-  constexpr int NF = 1 + 2 * L;
-  constexpr int EV = 16 / sizeof(T);
-  const int tid = threadIdx.x, nth = blockDim.x;
-  const bool fast = pl.vec_ok != 0 && pl.N % EV == 0;
-  float* cur = lds;
-  float* nxt = lds + nth * SLOT;
-
-  uint4 q[S / EV];
-  if (static_cast<int>(blockIdx.x) < nrows) {
-    const T* xrow = x + static_cast<size_t>(blockIdx.x) * pl.N;
-    if (fast) {
-      row1d_fetch<T, S>(xrow, pl.N, tid, nth, q);
-      row1d_commit<T, S, SLOT>(cur, pl.nl, tid, nth, q);
-    } else {
-      row1d_stage_scalar<T, S, SLOT>(xrow, cur, pl.N, pl.nl, tid, nth);
-    }
-  }
-  WT_LDS_BARRIER();
-  for (int rv = blockIdx.x; rv < nrows; rv += gridDim.x) {
-    const int row = WT_UNIFORM(rv);
-    const int c = row % pl.C;
-    const bool more = row + static_cast<int>(gridDim.x) < nrows;
-    const T* xnext = x + static_cast<size_t>(more ? row + gridDim.x : row) * pl.N;
-    wt_uniform_ptr fwc = (wt_uniform_ptr)(fw + static_cast<size_t>(c) * NF * K);
-    float* slot = cur + tid * SLOT;
-    float xs[S];
-    if (tid < pl.nl) {
-      row1d_read_slot<S>(slot, xs);
-    } else {
-#pragma unroll
-      for (int e = 0; e < S; ++e) xs[e] = 0.f;
-    }
-    if (fast && more) row1d_fetch<T, S>(xnext, pl.N, tid, nth, q);
-    RowPyramid<S, L> py;
-    row1d_analysis<S, L>(xs, py);
-    // the slot held this lane's samples only: it can take the lane's edges right away
-    row1d_publish<K, S, 0>(slot, xs);
-    row1d_publish_levels<K, S, L, 1>(slot, py);
-    WT_LDS_BARRIER();
-
-    float o[S];
-    {
-      const float bias = fb[c];
-#pragma unroll
-      for (int e = 0; e < S; ++e) o[e] = bias;
-      float ext[S + 2 * R];
-      row1d_extend<K, S, SLOT, 0>(cur, tid, nth, xs, ext);
-      row1d_conv<K, S>(ext, fwc, o);
-    }
-    float zc[S / 2];
-#pragma unroll
-    for (int e = 0; e < S / 2; ++e) zc[e] = 0.f;
-    row1d_synth<K, S, SLOT, L, L>(py, cur, tid, nth, fwc, zc, o);
-    WT_LDS_BARRIER();            // every neighbour has read this lane's edges
-    row1d_write_slot<S>(slot, o);
-    if (more) {                  // the other region is idle: nothing has read it since the last barrier but one
-      if (fast)
-        row1d_commit<T, S, SLOT>(nxt, pl.nl, tid, nth, q);
-      else
-        row1d_stage_scalar<T, S, SLOT>(xnext, nxt, pl.N, pl.nl, tid, nth);
-    }
-    WT_LDS_BARRIER();
-    row1d_unstage<T, S, SLOT>(out + static_cast<size_t>(row) * pl.N, cur, pl.N, pl.vec_ok != 0, tid, nth);
-    float* t = cur; cur = nxt; nxt = t;
   }
 }
 
@@ -473,27 +492,267 @@ __device__ __forceinline__ void row1d_wgrad_levels(const RowPyramid<S, L>& py, c
   if constexpr (l < L) row1d_wgrad_levels<K, S, SLOT, L, l + 1>(py, region, tid, nth, glo, acc);
 }
 
+// The per-chunk record of a workgroup's running sums: cross-lane sums, then cross-wave through `red`
+// ([waves][NRED] floats of LDS, idle by now), into partial[chunk][c][NF * K + 1].
+template <int K, int NF, bool SHARED = false>
+__device__ __forceinline__ void row1d_store_partial(const float (&acc)[NF][K], float gsum, float* __restrict__ red,
+                                                    float* __restrict__ dst, int tid, int nth) {
+  constexpr int NRED = NF * K + 1;
+  const int wave = tid >> 6, lane = tid & (kWave - 1);
+#pragma unroll
+  for (int f = 0; f < NF; ++f)
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const float v = wave_sum(acc[f][k]);
+      if (lane == 0) red[wave * NRED + f * K + k] = v;
+    }
+  {
+    const float v = wave_sum(gsum);
+    if (lane == 0) red[wave * NRED + NRED - 1] = v;
+  }
+  WT_LDS_BARRIER();
+  const int nwaves = nth >> 6;
+  for (int o = tid; o < NRED; o += nth) {
+    float v = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) v += red[wv * NRED + o];
+    if constexpr (SHARED) store_shared_f32(dst + o, v);
+    else dst[o] = v;
+  }
+}
+
+// Fused backward kernel, before the barrier: level l of a lane's pyramid from level l - 1 (`prev`), its edges
+// published at once; only the low-pass of the current level stays live (the levels are formed again, one at a time,
+// after the barrier: two operations per coefficient, against sixty registers for a whole pyramid).
+template <int K, int S, int L, int l>
+__device__ __forceinline__ void row1d_publish_chain(float* __restrict__ slot, const float (&prev)[(S >> (l - 1))]) {
+  constexpr int n = S >> l;
+  float lo[n], hi[n];
+#pragma unroll
+  for (int q = 0; q < n; ++q) {
+    lo[q] = (prev[2 * q] + prev[2 * q + 1]) * kInvSqrt2;
+    hi[q] = (prev[2 * q] - prev[2 * q + 1]) * kInvSqrt2;
+  }
+  row1d_publish<K, S, 1 + 2 * (l - 1)>(slot, lo);
+  row1d_publish<K, S, 2 + 2 * (l - 1)>(slot, hi);
+  if constexpr (l < L) row1d_publish_chain<K, S, L, l + 1>(slot, lo);
+}
+
+// Fused backward kernel, after the barrier: levels l..L of both halves of the backward pass, walking from the
+// finest level down.  `xprev` / `gprev` = low-pass of x / grad_out at level l - 1.  Per level: the four coefficient
+// arrays; the correlation sums of x's with grad_out's; the level's contribution to grad_x.  That contribution is
+// added to the samples directly: the inverse transform is linear, and a reconstruction with zero detail below level
+// l is the level-l result repeated 2^(l-1) times and scaled by 2^(-(l-1)/2), so the levels need not be visited
+// coarsest first and no level's coefficients outlive its visit.
+template <int K, int S, int SLOT, int L, int l>
+__device__ __forceinline__ void row1d_bwd_levels(const float* __restrict__ xregion, const float* __restrict__ gregion,
+                                                 int tid, int nth, const RowWeights<K, L>& fwc,
+                                                 const float (&xprev)[(S >> (l - 1))],
+                                                 const float (&gprev)[(S >> (l - 1))], float (&acc)[1 + 2 * L][K],
+                                                 float (&o)[S]) {
+  constexpr int R = K / 2;
+  constexpr int n = S >> l;
+  constexpr int A = 1 + 2 * (l - 1);
+  float xlo[n], glo[n], ylo[n], yhi[n];
+#pragma unroll
+  for (int q = 0; q < n; ++q) { ylo[q] = 0.f; yhi[q] = 0.f; }
+  {
+    float xhi[n], ghi[n];
+#pragma unroll
+    for (int q = 0; q < n; ++q) {
+      xlo[q] = (xprev[2 * q] + xprev[2 * q + 1]) * kInvSqrt2;
+      xhi[q] = (xprev[2 * q] - xprev[2 * q + 1]) * kInvSqrt2;
+      glo[q] = (gprev[2 * q] + gprev[2 * q + 1]) * kInvSqrt2;
+      ghi[q] = (gprev[2 * q] - gprev[2 * q + 1]) * kInvSqrt2;
+    }
+    {
+      float ext[n + 2 * R];
+      row1d_extend<K, S, SLOT, A + 1>(xregion, tid, nth, xhi, ext);
+      row1d_corr<K, n>(ext, ghi, acc[A + 1]);
+    }
+    {
+      float ext[n + 2 * R];
+      row1d_extend<K, S, SLOT, A + 1>(gregion, tid, nth, ghi, ext);
+      row1d_conv<K, L, A + 1, n>(ext, fwc, yhi);
+    }
+    pin_values(yhi);
+    WT_CHUNK_FENCE();      // (the edge reads of the next part stay below: one part's edges live at a time)
+  }
+  {
+    float ext[n + 2 * R];
+    row1d_extend<K, S, SLOT, A>(xregion, tid, nth, xlo, ext);
+    row1d_corr<K, n>(ext, glo, acc[A]);
+  }
+  {
+    float ext[n + 2 * R];
+    row1d_extend<K, S, SLOT, A>(gregion, tid, nth, glo, ext);
+    row1d_conv<K, L, A, n>(ext, fwc, ylo);
+  }
+  // one inverse butterfly (1/sqrt2), then l - 1 repeats (1/sqrt2 each)
+  float scale = kInvSqrt2;
+#pragma unroll
+  for (int i = 1; i < l; ++i) scale *= kInvSqrt2;
+  constexpr int REP = 1 << (l - 1);
+#pragma unroll
+  for (int q = 0; q < n; ++q) {
+    const float ev = (ylo[q] + yhi[q]) * scale, od = (ylo[q] - yhi[q]) * scale;
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+      o[(2 * q) * REP + r] += ev;
+      o[(2 * q + 1) * REP + r] += od;
+    }
+  }
+  pin_values(o);
+  WT_CHUNK_FENCE();
+  if constexpr (l < L) row1d_bwd_levels<K, S, SLOT, L, l + 1>(xregion, gregion, tid, nth, fwc, xlo, glo, acc, o);
+}
+
+// The forward / input-gradient kernel's walk over the levels, finest first, on the same terms: per level the two
+// coefficient arrays, their convolutions, and the level's contribution added to the samples directly.
+template <int K, int S, int SLOT, int L, int l>
+__device__ __forceinline__ void row1d_fwd_levels(const RowEdges<K, L>& ed, const RowWeights<K, L>& fwc,
+                                                 const float (&xprev)[(S >> (l - 1))], float (&o)[S]) {
+  constexpr int R = K / 2;
+  constexpr int n = S >> l;
+  constexpr int A = 1 + 2 * (l - 1);
+  float xlo[n], ylo[n], yhi[n];
+#pragma unroll
+  for (int q = 0; q < n; ++q) { ylo[q] = 0.f; yhi[q] = 0.f; }
+  {
+    float xhi[n];
+#pragma unroll
+    for (int q = 0; q < n; ++q) {
+      xlo[q] = (xprev[2 * q] + xprev[2 * q + 1]) * kInvSqrt2;
+      xhi[q] = (xprev[2 * q] - xprev[2 * q + 1]) * kInvSqrt2;
+    }
+    float ext[n + 2 * R];
+    row1d_extend_with<K, S, L, A + 1>(ed, xhi, ext);
+    row1d_conv<K, L, A + 1, n>(ext, fwc, yhi);
+  }
+  {
+    float ext[n + 2 * R];
+    row1d_extend_with<K, S, L, A>(ed, xlo, ext);
+    row1d_conv<K, L, A, n>(ext, fwc, ylo);
+  }
+  float scale = kInvSqrt2;
+#pragma unroll
+  for (int i = 1; i < l; ++i) scale *= kInvSqrt2;
+  constexpr int REP = 1 << (l - 1);
+#pragma unroll
+  for (int q = 0; q < n; ++q) {
+    const float ev = (ylo[q] + yhi[q]) * scale, od = (ylo[q] - yhi[q]) * scale;
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+      o[(2 * q) * REP + r] += ev;
+      o[(2 * q + 1) * REP + r] += od;
+    }
+  }
+  if constexpr (l < L) row1d_fwd_levels<K, S, SLOT, L, l + 1>(ed, fwc, xlo, o);
+}
+
+// Forward / input-gradient kernel.  grid = (channels, batch chunks), block = lanes (multiple of 64,
+// >= ceil(N / S)), dynamic LDS = one slot region (row1d_region floats).  A workgroup walks the rows (b, c) of
+// its chunk of batch items; the next row is fetched into registers while the current one is computed and
+// committed to the slots once the current outputs have left them.  One region instead of two alternating
+// ones: half the LDS per workgroup, i.e. twice the workgroups per CU, which pays more here than the two
+// barriers per row it costs.  flip != 0: the input gradient (taps reversed, no bias).
+template <typename T, int K, int L, int S>
+__global__ __launch_bounds__(kRow1dMaxLanes) void wt1d_row_kernel(const T* __restrict__ x, T* __restrict__ out,
+                                                                   const ParamTable prm, int pdtype, int flip,
+                                                                   Row1D pl, int B, int per_chunk) {
+  WT_SHARED_FLOATS(lds);
+  constexpr int R = K / 2;
+  constexpr int SLOT = row1d_slot(K, L, S);
+  constexpr int EV = 16 / sizeof(T);
+  const int tid = threadIdx.x, nth = blockDim.x;
+  const int c = blockIdx.x;
+  const int b_begin = static_cast<int>(blockIdx.y) * per_chunk;
+  const int b_end = b_begin + per_chunk < B ? b_begin + per_chunk : B;
+  const bool fast = pl.vec_ok != 0 && pl.N % EV == 0;
+  constexpr int G = row1d_guard(K, L, S);
+  float* cur = lds + G * SLOT;                      // (the region points at the slot of lane 0, behind its left guard)
+  row1d_zero_guards<K, L, S>(lds, 1, tid, nth);
+  auto row_of = [&](int b) { return (static_cast<size_t>(b) * pl.C + c) * pl.N; };
+
+  uint4 q[S / EV];
+  if (b_begin < b_end && fast) row1d_fetch<T, S>(x + row_of(b_begin), pl.N, tid, nth, q);
+  RowWeights<K, L> fwc;                 // (its parameter loads share the latency of the first row's)
+  row1d_fold<K, L>(prm, pdtype, c, flip, fwc);
+  const float bias = (!flip && prm.base_bias != nullptr)
+                         ? load_param(prm.base_bias, pdtype, c) * load_param(prm.base_scale, pdtype, c) : 0.f;
+  if (b_begin < b_end) {
+    if (fast)
+      row1d_commit<T, S, SLOT>(cur, pl.nl, tid, nth, q);
+    else
+      row1d_stage_scalar<T, S, SLOT>(x + row_of(b_begin), cur, pl.N, pl.nl, tid, nth);
+  }
+  WT_LDS_BARRIER();
+  for (int bv = b_begin; bv < b_end; ++bv) {
+    const int b = WT_UNIFORM(bv);
+    const bool more = b + 1 < b_end;
+    const T* xnext = x + row_of(more ? b + 1 : b);
+    float* slot = cur + tid * SLOT;
+    float xs[S];
+    if (tid < pl.nl) {
+      row1d_read_slot<S>(slot, xs);
+    } else {
+#pragma unroll
+      for (int e = 0; e < S; ++e) xs[e] = 0.f;
+    }
+    if (fast && more) row1d_fetch<T, S>(xnext, pl.N, tid, nth, q);
+    // the slot held this lane's samples only: it can take the lane's edges right away
+    row1d_publish<K, S, 0>(slot, xs);
+    row1d_publish_chain<K, S, L, 1>(slot, xs);
+    WT_LDS_BARRIER();
+    pin_values(xs);              // (the levels are formed again below, one at a time, not kept across the barrier)
+
+    RowEdges<K, L> ed;
+    row1d_load_edges<K, S, SLOT, L>(cur, tid, ed);
+    float o[S];
+    {
+#pragma unroll
+      for (int e = 0; e < S; ++e) o[e] = bias;
+      float ext[S + 2 * R];
+      row1d_extend_with<K, S, L, 0>(ed, xs, ext);
+      row1d_conv<K, L, 0, S>(ext, fwc, o);
+    }
+    row1d_fwd_levels<K, S, SLOT, L, 1>(ed, fwc, xs, o);
+    WT_LDS_BARRIER();            // every neighbour has read this lane's edges
+    row1d_write_slot<S>(slot, o);
+    WT_LDS_BARRIER();
+    row1d_unstage<T, S, SLOT>(out + row_of(b), cur, pl.N, pl.vec_ok != 0, tid, nth);
+    WT_LDS_BARRIER();            // the outputs have left the slots
+    if (more) {
+      if (fast)
+        row1d_commit<T, S, SLOT>(cur, pl.nl, tid, nth, q);
+      else
+        row1d_stage_scalar<T, S, SLOT>(xnext, cur, pl.N, pl.nl, tid, nth);
+    }
+    WT_LDS_BARRIER();
+  }
+}
+
 // Parameter gradients, first stage.  grid = (C, nchunk), block = lanes, dynamic LDS =
 // 2 * block * SLOT floats (x slots, then grad_out slots).  A workgroup walks `per_chunk` rows
 // of one channel; every lane keeps K sums per filter in registers.  Output layout as the
 // tiled kernel: partial[chunk][c][(1 + 2L) * K + 1].
-template <typename T, int K, int L>
+template <typename T, int K, int L, int S>
 __global__ __launch_bounds__(kRow1dMaxLanes) void wt1d_row_wgrad_kernel(const T* __restrict__ x,
                                                                          const T* __restrict__ g,
                                                                          float* __restrict__ partial, Row1D pl,
                                                                          int B, int per_chunk) {
   WT_SHARED_FLOATS(lds);
   constexpr int R = K / 2;
-  constexpr int S = row1d_samples(K, L);
-  constexpr int SLOT = row1d_slot(K, L);
+  constexpr int SLOT = row1d_slot(K, L, S);
   constexpr int NF = 1 + 2 * L;
   const int c = blockIdx.x;
   const int chunk = blockIdx.y;
   const int tid = threadIdx.x, nth = blockDim.x;
-  float* xlds = lds;
-  float* glds = lds + nth * SLOT;
+  constexpr int G = row1d_guard(K, L, S);
+  float* xlds = lds + G * SLOT;                     // (regions point at the slot of lane 0, behind their left guard)
+  float* glds = xlds + (nth + 2 * G) * SLOT;
   float* slot = xlds + tid * SLOT;
   const float* gslot = glds + tid * SLOT;
+  row1d_zero_guards<K, L, S>(lds, 2, tid, nth);
 
   constexpr int EV = 16 / sizeof(T);
   const bool fast = pl.vec_ok != 0 && pl.N % EV == 0;
@@ -540,26 +799,149 @@ __global__ __launch_bounds__(kRow1dMaxLanes) void wt1d_row_wgrad_kernel(const T*
   }
 
   constexpr int NRED = NF * K + 1;
-  float* red = lds;              // [waves][NRED]
-  const int wave = tid >> 6, lane = tid & (kWave - 1);
+  row1d_store_partial<K, NF>(acc, gsum, lds, partial + (static_cast<size_t>(chunk) * pl.C + c) * NRED, tid, nth);
+}
+
+constexpr int kRow1dBwdMaxLanes = 256;      // threads per workgroup of the fused backward kernel (register budget)
+// (K, L) pairs the fused backward kernel is built for: its (1 + 2L) * K + 1 running sums per lane must leave room for
+// the rest in 256 registers (beyond 50 sums, 45 with 32 samples per lane, the compiler spills; those pairs run the
+// backward pass as two kernels).
+constexpr bool row1d_bwd_built(int K, int L, int S) {
+  return row1d_built(K, L, S) && (1 + 2 * L) * K <= (S == 16 ? 50 : 45);
+}
+
+// The whole backward pass of a row-resident shape in one kernel.  grid = (C, nchunk), block = lanes, dynamic LDS =
+// 2 * block * SLOT floats (x slots, then grad_out slots, which also stage grad_x on its way out).  Per row: x and
+// grad_out are read once; grad_x = the layer applied to grad_out with reversed taps and no bias; the correlation
+// sums of x's pyramid with grad_out's go into (1 + 2L) * K + 1 running sums per lane.  After its rows a workgroup
+// stores its record of sums and draws its channel's ticket; the last one of a channel runs the second stage
+// (wgrad_finish_channel) for it and leaves the ticket zero.  `tickets`: C words, zero at launch.
+template <typename T, int K, int L, int S>
+__global__ __launch_bounds__(kRow1dBwdMaxLanes, 2) void wt1d_row_bwd_kernel(const T* __restrict__ x,
+                                                                          const T* __restrict__ g,
+                                                                          T* __restrict__ gx,
+                                                                          float* __restrict__ partial,
+                                                                          unsigned* __restrict__ tickets,
+                                                                          const ParamTable prm, int pdtype,
+                                                                          const GradTable gt, Row1D pl, int B,
+                                                                          int per_chunk, int nchunk) {
+  WT_SHARED_FLOATS(lds);
+  constexpr int R = K / 2;
+  constexpr int SLOT = row1d_slot(K, L, S);
+  constexpr int NF = 1 + 2 * L;
+  constexpr int EV = 16 / sizeof(T);
+  const int c = blockIdx.x;
+  const int chunk = blockIdx.y;
+  const int tid = threadIdx.x, nth = blockDim.x;
+  constexpr int G = row1d_guard(K, L, S);
+  float* xlds = lds + G * SLOT;                     // (regions point at the slot of lane 0, behind their left guard)
+  float* glds = xlds + (nth + 2 * G) * SLOT;
+  float* xslot = xlds + tid * SLOT;
+  float* gslot = glds + tid * SLOT;
+  row1d_zero_guards<K, L, S>(lds, 2, tid, nth);
+  const bool fast = pl.vec_ok != 0 && pl.N % EV == 0;
+
+  RowWeights<K, L> fwc;
+  row1d_fold<K, L>(prm, pdtype, c, 1, fwc);
+
+  float acc[NF][K];
+  float gsum = 0.f;
 #pragma unroll
   for (int f = 0; f < NF; ++f)
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const float v = wave_sum(acc[f][k]);
-      if (lane == 0) red[wave * NRED + f * K + k] = v;
+    for (int k = 0; k < K; ++k) acc[f][k] = 0.f;
+
+  const int b_end = (chunk + 1) * per_chunk < B ? (chunk + 1) * per_chunk : B;
+  // with 16 samples per lane, rows on the fast path (16-byte sized and aligned) are fetched one row ahead into
+  // registers; with 32 the registers for that are not there, and the rows are staged as the loop reaches them
+  constexpr bool kAhead = S <= 16;
+  const bool ahead = kAhead && fast;
+  uint4 qx[kAhead ? S / EV : 1], qg[kAhead ? S / EV : 1];
+  const int b_first = chunk * per_chunk;
+  if (b_first < b_end && ahead) {
+    const size_t r0 = (static_cast<size_t>(b_first) * pl.C + c) * pl.N;
+    if constexpr (kAhead) {
+      row1d_fetch<T, S>(x + r0, pl.N, tid, nth, qx);
+      row1d_fetch<T, S>(g + r0, pl.N, tid, nth, qg);
+      row1d_commit<T, S, SLOT>(xlds, pl.nl, tid, nth, qx);
+      row1d_commit<T, S, SLOT>(glds, pl.nl, tid, nth, qg);
     }
-  {
-    const float v = wave_sum(gsum);
-    if (lane == 0) red[wave * NRED + NRED - 1] = v;
   }
-  WT_LDS_BARRIER();
-  float* dst = partial + (static_cast<size_t>(chunk) * pl.C + c) * NRED;
-  const int nwaves = nth >> 6;
-  for (int o = tid; o < NRED; o += nth) {
-    float v = 0.f;
-    for (int wv = 0; wv < nwaves; ++wv) v += red[wv * NRED + o];
-    dst[o] = v;
+  for (int bv = b_first; bv < b_end; ++bv) {
+    const int b = WT_UNIFORM(bv);
+    const size_t roff = (static_cast<size_t>(b) * pl.C + c) * pl.N;
+    const bool more = b + 1 < b_end;
+    const size_t rnext = (static_cast<size_t>(more ? b + 1 : b) * pl.C + c) * pl.N;
+    if (!ahead) {
+      if (fast) {
+        row1d_stage_pair<T, S, SLOT>(x + roff, g + roff, xlds, glds, pl.N, pl.nl, tid, nth);
+      } else {
+        row1d_stage_scalar<T, S, SLOT>(x + roff, xlds, pl.N, pl.nl, tid, nth);
+        row1d_stage_scalar<T, S, SLOT>(g + roff, glds, pl.N, pl.nl, tid, nth);
+      }
+    }
+    WT_LDS_BARRIER();
+    float xs[S], gs[S];
+    if (tid < pl.nl) {
+      row1d_read_slot<S>(xslot, xs);
+      row1d_read_slot<S>(gslot, gs);
+    } else {
+#pragma unroll
+      for (int q = 0; q < S; ++q) { xs[q] = 0.f; gs[q] = 0.f; }
+    }
+    if constexpr (kAhead) {
+      if (ahead && more) {
+        row1d_fetch<T, S>(x + rnext, pl.N, tid, nth, qx);
+        row1d_fetch<T, S>(g + rnext, pl.N, tid, nth, qg);
+      }
+    }
+    row1d_publish<K, S, 0>(xslot, xs);
+    row1d_publish<K, S, 0>(gslot, gs);
+    row1d_publish_chain<K, S, L, 1>(xslot, xs);
+    row1d_publish_chain<K, S, L, 1>(gslot, gs);
+    WT_LDS_BARRIER();
+    // (opaque from here on: otherwise the compiler keeps the coefficients it formed for the edges above alive across
+    // the barrier instead of forming them again level by level)
+    pin_values(xs);
+    pin_values(gs);
+    // base conv: its correlation sums, and its share of grad_x (the layer on grad_out with the reversed taps)
+    float o[S];
+#pragma unroll
+    for (int e = 0; e < S; ++e) o[e] = 0.f;
+    {
+      float ext[S + 2 * R];
+      row1d_extend<K, S, SLOT, 0>(xlds, tid, nth, xs, ext);
+      row1d_corr<K, S>(ext, gs, acc[0]);
+#pragma unroll
+      for (int q = 0; q < S; ++q) gsum += gs[q];
+    }
+    {
+      float ext[S + 2 * R];
+      row1d_extend<K, S, SLOT, 0>(glds, tid, nth, gs, ext);
+      row1d_conv<K, L, 0, S>(ext, fwc, o);
+    }
+    pin_values(o);
+    WT_CHUNK_FENCE();
+    row1d_bwd_levels<K, S, SLOT, L, 1>(xlds, glds, tid, nth, fwc, xs, gs, acc, o);
+    WT_LDS_BARRIER();            // every neighbour has read this lane's edges
+    row1d_write_slot<S>(gslot, o);
+    WT_LDS_BARRIER();
+    row1d_unstage<T, S, SLOT>(gx + roff, glds, pl.N, pl.vec_ok != 0, tid, nth);
+    WT_LDS_BARRIER();            // the next row's staging overwrites the slots read above
+    if constexpr (kAhead) {
+      if (ahead && more) {
+        row1d_commit<T, S, SLOT>(xlds, pl.nl, tid, nth, qx);
+        row1d_commit<T, S, SLOT>(glds, pl.nl, tid, nth, qg);
+      }
+    }
+  }
+
+  constexpr int NRED = NF * K + 1;
+  row1d_store_partial<K, NF, true>(acc, gsum, lds, partial + (static_cast<size_t>(chunk) * pl.C + c) * NRED, tid, nth);
+  unsigned* flag = reinterpret_cast<unsigned*>(lds + (nth >> 6) * NRED);
+  if (workgroup_is_last(tickets + c, static_cast<unsigned>(nchunk), flag)) {
+    wgrad_finish_channel<true>(partial, nchunk, prm, pdtype, gt, pl.C, c, 2, L, K, lds);
+    if (tid == 0) tickets[c] = 0u;
   }
 }
 

@@ -1076,27 +1076,47 @@ __global__ __launch_bounds__(512, 4) void wt2d_wgrad_kernel(const T* __restrict_
 // Second stage: sum the per-chunk partials and apply the chain rule of the folding
 //   dw = gamma * dWt,  dgamma = sum_t w * dWt (+ bias * sumG for the base scale),
 //   dbias = gamma_b * sumG        (cf. fast_wtconv/cuda_haar/haar_cuda.py:168-197,657-676)
-// One workgroup per channel, one thread per (filter, tap) plus one for sumG (a single pass when the workgroup has
-// NF*KK + 1 threads: the kernel is a chain of load latencies, nothing else); the per-filter dot products go
-// through LDS.  S = 4 (2-D) or 2 (1-D).  blockDim.x >= NF, dynamic LDS NF*KK + 1 floats.
-__global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchunk, ParamTable p,
-                                    int pdtype, GradTable gt, int C, int S, int L, int KK) {
-  WT_SHARED_FLOATS(prod);
+// for one channel, by the threads of one workgroup: one thread per (filter, tap) plus one for sumG where the
+// workgroup has that many (else strided); the per-filter dot products go through `prod` (NF*KK + 1 floats of
+// LDS).  S = 4 (2-D) or 2 (1-D).  blockDim.x >= NF.  The chunks are summed in index order whichever workgroup
+// runs this, so the result does not depend on the order in which the first stage finished.  SHARED: called by the
+// last workgroup of a first stage that finishes its channels itself: the records of the other workgroups are read
+// with load_shared_f32.
+template <bool SHARED>
+__device__ __forceinline__ void wgrad_finish_channel(const float* __restrict__ partial, int nchunk,
+                                                     const ParamTable& p, int pdtype, const GradTable& gt, int C,
+                                                     int c, int S, int L, int KK, float* __restrict__ prod) {
   const int NF = 1 + S * L;
   const int stride = NF * KK + 1;
-  const int c = blockIdx.x;
+  // table entries of a level picked with constant indices (a per-lane index into the argument structs would send
+  // them to scratch memory)
+  auto level_w = [&](int l) { const void* q = p.wt_weight[0];
+#pragma unroll
+    for (int i = 1; i < kMaxLevels; ++i) q = l == i ? p.wt_weight[i] : q; return q; };
+  auto level_s = [&](int l) { const void* q = p.wt_scale[0];
+#pragma unroll
+    for (int i = 1; i < kMaxLevels; ++i) q = l == i ? p.wt_scale[i] : q; return q; };
+  auto grad_w = [&](int l) { float* q = gt.wt_weight[0];
+#pragma unroll
+    for (int i = 1; i < kMaxLevels; ++i) q = l == i ? gt.wt_weight[i] : q; return q; };
+  auto grad_s = [&](int l) { float* q = gt.wt_scale[0];
+#pragma unroll
+    for (int i = 1; i < kMaxLevels; ++i) q = l == i ? gt.wt_scale[i] : q; return q; };
   for (int o = threadIdx.x; o <= NF * KK; o += blockDim.x) {      // (the last index is the sumG slot of the records)
     const bool tap = o < NF * KK;
     const int f = tap ? o / KK : 0, t = tap ? o - f * KK : 0;
     const int l = f == 0 ? 0 : (f - 1) / S, chn = f == 0 ? c : c * S + (f - 1) % S;
     // parameters first: their loads overlap those of the partial sums
-    const float gam = load_param(f == 0 ? p.base_scale : p.wt_scale[l], pdtype, chn);
-    const float wv = load_param(f == 0 ? p.base_weight : p.wt_weight[l], pdtype, chn * KK + t);
+    const float gam = load_param(f == 0 ? p.base_scale : level_s(l), pdtype, chn);
+    const float wv = load_param(f == 0 ? p.base_weight : level_w(l), pdtype, chn * KK + t);
     float sum = 0.f;
 #pragma unroll 8                       // several chunk loads in flight; the order of the adds is unchanged
-    for (int ch = 0; ch < nchunk; ++ch) sum += partial[(static_cast<size_t>(ch) * C + c) * stride + o];
+    for (int ch = 0; ch < nchunk; ++ch) {
+      const float* src = partial + (static_cast<size_t>(ch) * C + c) * stride + o;
+      sum += SHARED ? load_shared_f32(src) : *src;
+    }
     if (tap) {
-      float* dst = f == 0 ? gt.base_weight : gt.wt_weight[l];
+      float* dst = f == 0 ? gt.base_weight : grad_w(l);
       dst[chn * KK + t] = gam * sum;
       prod[o] = wv * sum;
     } else {
@@ -1117,9 +1137,23 @@ __global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchun
       gt.base_scale[c] = dot;
     } else {
       const int l = (o - 1) / S, chn = c * S + (o - 1) % S;
-      gt.wt_scale[l][chn] = dot;
+      grad_s(l)[chn] = dot;
     }
   }
+}
+
+// The second stage as a launch of its own (one workgroup per channel, dynamic LDS NF*KK + 1 floats): after a first
+// stage that does not finish its channels itself.
+__global__ void wgrad_finish_kernel(const float* __restrict__ partial, int nchunk, ParamTable p,
+                                    int pdtype, GradTable gt, int C, int S, int L, int KK) {
+  WT_SHARED_FLOATS(prod);
+  wgrad_finish_channel<false>(partial, nchunk, p, pdtype, gt, C, static_cast<int>(blockIdx.x), S, L, KK, prod);
+}
+
+// Clears the ticket words of a first stage that finishes its channels itself (a kernel rather than a memset, so
+// that a caller may record the call into a HIP graph).
+__global__ void zero_tickets_kernel(unsigned* __restrict__ t, int n) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) t[i] = 0u;
 }
 
 }  // namespace wt

@@ -14,6 +14,8 @@
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <torch/csrc/autograd/function.h>
+#include <torch/csrc/autograd/functions/basic_ops.h>
 
 #include <optional>
 #include <vector>
@@ -199,7 +201,23 @@ class WTConvNode : public torch::autograd::Function<WTConvNode> {
         rc = abi.bwdpar1(x.data_ptr(), g.data_ptr(), &p, &gt, s.B, s.C, s.W, K, L, dt, pdt, ws.data_ptr(), wsz, stream);
     }
     if (rc) fail(rc, "wtconv backward");
+    // The gradients come from raw pointers and carry no graph.  Under create_graph=True every result that something
+    // differentiable went into gets a node that raises when it is differentiated (what once_differentiable does for
+    // the Python function): a second-order term is refused instead of being treated as a constant.
+    bool twice = false;
+    if (at::GradMode::is_enabled()) {
+      twice = grad_outputs[0].requires_grad();
+      for (const Tensor& t : saved) twice = twice || (t.defined() && t.requires_grad());
+    }
+    auto refuse = [&](Tensor& t) {
+      if (!twice || !t.defined()) return;
+      auto err = std::make_shared<torch::autograd::Error>(
+          "the backward pass of the WTConv layer is not differentiable (double backward / create_graph=True through "
+          "this layer is not supported)", torch::autograd::edge_list());
+      torch::autograd::create_gradient_edge(t, err);
+    };
     res[0] = grad_x;
+    refuse(res[0]);
     if (need_params) {
       if (!f32) {
         const Tensor cast = flat.to(base_w.scalar_type());
@@ -216,6 +234,7 @@ class WTConvNode : public torch::autograd::Function<WTConvNode> {
       res[2] = views[1];
       res[3] = views[2];
       for (int i = 0; i < 2 * L; ++i) res[4 + i] = views[3 + i];
+      for (int i = 1; i < 4 + 2 * L; ++i) refuse(res[i]);
     }
     return res;
   }

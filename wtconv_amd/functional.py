@@ -244,14 +244,33 @@ class _WTConvFn(torch.autograd.Function):
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable      # double backward raises instead of being silently wrong
     def backward(ctx, grad_out):
         x, base_w, base_b, base_s, *wt = ctx.saved_tensors
         dims, K, L = ctx.dims, ctx.K, ctx.L
         need_params = any(ctx.needs_input_grad[i] for i in (1, 2, 3)) or any(ctx.needs_input_grad[7:])
-        grad_x, grads = _backward_impl(grad_out, x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L,
-                                       ctx.needs_input_grad[0], need_params, ctx.tabinfo)
-        return (grad_x, grads[0], grads[1], grads[2], None, None, None, *grads[3:])
+        # Under create_graph=True a second-order term through this layer is refused, not dropped: the gradients come
+        # from raw pointers and carry no graph, so every result that something differentiable went into (the upstream
+        # gradient or any saved tensor -- once_differentiable looks at the upstream gradient only) gets a node that
+        # raises when it is differentiated.
+        twice = torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad for t in (grad_out, x, base_w, base_b, base_s, *wt))
+        with torch.no_grad():
+            grad_x, grads = _backward_impl(grad_out, x, base_w, base_b, base_s, wt[:L], wt[L:], dims, K, L,
+                                           ctx.needs_input_grad[0], need_params, ctx.tabinfo)
+        res = (grad_x, grads[0], grads[1], grads[2], None, None, None, *grads[3:])
+        if twice:
+            res = _refuse_second_order(res)
+        return res
+
+
+def _refuse_second_order(outputs):
+    err = torch._C._functions.DelayedError(
+        b"the backward pass of the WTConv layer is not differentiable (double backward / create_graph=True through "
+        b"this layer is not supported)", len(outputs))
+
+    def fake(v):      # an input that requires grad makes DelayedError attach its raising node to the matching output
+        return v.detach().requires_grad_(True) if v is not None else None
+    return err(*[fake(v) for v in outputs])
 
 
 # ---------------------------------------------------------------------------------------------

@@ -95,12 +95,17 @@ class WTConvNeXtBlock(nn.Module):
                 and ops.usable(shortcut)):
             # inference on the GPU: NCHW -> LayerNorm -> NHWC, and NHWC -> layer scale -> + shortcut -> NCHW, are one
             # kernel each instead of a layout copy plus an elementwise pass each
-            x = ops.channel_norm(x, self.norm.weight, self.norm.bias, self.norm.eps, nhwc=True)
-            x = self.mlp(x)
-            return ops.block_residual(x.contiguous(), shortcut, self.gamma)
-        x = x.permute(0, 2, 3, 1)
-        x = self.mlp(self.norm(x))
-        x = x.permute(0, 3, 1, 2)
+            y = self.mlp(ops.channel_norm(x, self.norm.weight, self.norm.bias, self.norm.eps, nhwc=True))
+            # the MLP may still record for autograd (its own parameters can be trainable while everything before it
+            # is frozen) or change the dtype; the residual kernel takes raw pointers, so only a plain tensor of the
+            # shortcut's type goes there
+            if ops.usable_nhwc(y, shortcut):
+                return ops.block_residual(y.contiguous(), shortcut, self.gamma)
+            x = y.permute(0, 3, 1, 2)
+        else:
+            x = x.permute(0, 2, 3, 1)
+            x = self.mlp(self.norm(x))
+            x = x.permute(0, 3, 1, 2)
         if self.gamma is not None:
             x = x.mul(self.gamma.reshape(1, -1, 1, 1))
         return self.drop_path(x) + shortcut
