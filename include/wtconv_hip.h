@@ -28,7 +28,7 @@ extern "C" {
 #endif
 
 #define WTCONV_MAX_LEVELS 5
-#define WTCONV_ABI_VERSION 4
+#define WTCONV_ABI_VERSION 5
 
 enum { WTCONV_F32 = 0, WTCONV_BF16 = 1, WTCONV_F16 = 2 };
 
@@ -165,7 +165,7 @@ int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const w
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- the passes of a WTConvNeXt block around its WTConv layer, each as one kernel that transposes through LDS.
- * Forward only (inference); activations in `dtype`, weight / bias / gamma in `param_dtype`; C must be even.
+ * Activations in `dtype` (float or bfloat16), weight / bias / gamma in `param_dtype`; C must be even.
  *
  * wtconv_channel_norm: LayerNorm over the channels of every pixel of x (B, C, HW), biased variance, `eps` inside
  * the square root.  out_nhwc != 0 writes (B, HW, C): the permute to NHWC followed by nn.LayerNorm that the block
@@ -180,6 +180,26 @@ int wtconv_channel_norm(const void* x, void* out, const void* weight, const void
  * scale).  out may be the shortcut itself. */
 int wtconv_block_residual(const void* y, const void* shortcut, const void* gamma, void* out, int B, int C, int HW,
                           int dtype, int param_dtype, void* stream);
+
+/* ---- the same two passes under autograd (training keeps the block's structure,
+ * wtconvnext/wtconvnext.py:125-140; in the reference these gradients come from autograd through
+ * permute / nn.LayerNorm / mul / add).  Parameter gradients are written as float; the workspace
+ * (wtconv_block_workspace_bytes(...) bytes, 4-byte aligned) takes per-workgroup partial sums that a
+ * second small kernel adds up in a fixed order (no atomics). */
+size_t wtconv_block_workspace_bytes(int B, int C, int HW, int dtype);
+
+/* Backward of wtconv_channel_norm: x (B, C, HW) is the forward input, dy the gradient of the forward
+ * output ((B, HW, C) if dy_nhwc != 0, else (B, C, HW)); writes dx (B, C, HW), dweight (C), dbias (C). */
+int wtconv_channel_norm_backward(const void* x, const void* dy, const void* weight, void* dx, float* dweight,
+                                 float* dbias, int B, int C, int HW, float eps, int dtype, int param_dtype,
+                                 int dy_nhwc, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward of wtconv_block_residual with a layer scale: dout (B, C, HW) is the gradient of the block's
+ * output (the shortcut's gradient is dout itself), y (B, HW, C) the forward's NHWC input; writes
+ * dy (B, HW, C) = gamma[c] * dout and dgamma (C) = sum dout * y. */
+int wtconv_block_residual_backward(const void* dout, const void* y, const void* gamma, void* dy, float* dgamma,
+                                   int B, int C, int HW, int dtype, int param_dtype, void* workspace,
+                                   size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

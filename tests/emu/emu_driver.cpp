@@ -82,6 +82,43 @@ int main(int argc, char** argv) {
     fclose(fo);
     return 0;
   }
+  if (dims == 3 || dims == 4) {
+    // block passes: header {dims, B, C, H, W, nhwc (K slot), unused, dtype, pdtype, unused}
+    //   dims == 3: in x, dy, weight, bias            -> out, dx, dweight, dbias       (channel norm, forward + backward)
+    //   dims == 4: in y (NHWC), shortcut, gamma, dout -> out, dy (NHWC), dgamma        (block residual, forward + backward)
+    const int HW = H * W, nhwc = K;
+    const size_t P = static_cast<size_t>(B) * C * HW;
+    Buf a0 = read_buf(fp, P, dtype), a1 = read_buf(fp, P, dtype);
+    Buf p0 = read_buf(fp, C, pdtype);
+    Buf p1 = dims == 3 ? read_buf(fp, C, pdtype) : read_buf(fp, P, dtype);
+    fclose(fp);
+    Buf o0 = out_buf(P, dtype), o1 = out_buf(P, dtype);
+    std::vector<float> g0(C, -777.f), g1(C, -777.f);
+    std::vector<char> ws(wtconv_block_workspace_bytes(B, C, HW, dtype));
+    int rc;
+    if (dims == 3) {
+      rc = wtconv_channel_norm(a0.ptr(), o0.ptr(), p0.ptr(), p1.ptr(), B, C, HW, 1e-6f, dtype, pdtype, nhwc, nullptr);
+      if (rc) { fprintf(stderr, "channel_norm: %s\n", wtconv_last_error()); return 3; }
+      rc = wtconv_channel_norm_backward(a0.ptr(), a1.ptr(), p0.ptr(), o1.ptr(), g0.data(), g1.data(), B, C, HW, 1e-6f, dtype,
+                                        pdtype, nhwc, ws.data(), ws.size(), nullptr);
+      if (rc) { fprintf(stderr, "channel_norm_backward: %s\n", wtconv_last_error()); return 3; }
+    } else {
+      rc = wtconv_block_residual(a0.ptr(), a1.ptr(), p0.ptr(), o0.ptr(), B, C, HW, dtype, pdtype, nullptr);
+      if (rc) { fprintf(stderr, "block_residual: %s\n", wtconv_last_error()); return 3; }
+      rc = wtconv_block_residual_backward(p1.ptr(), a0.ptr(), p0.ptr(), o1.ptr(), g0.data(), B, C, HW, dtype, pdtype,
+                                          ws.data(), ws.size(), nullptr);
+      if (rc) { fprintf(stderr, "block_residual_backward: %s\n", wtconv_last_error()); return 3; }
+    }
+    o0.unpack(); o1.unpack();
+    FILE* fo = fopen(argv[2], "wb");
+    if (!fo) { perror("open out"); return 2; }
+    fwrite(o0.f.data(), 4, P, fo);
+    fwrite(o1.f.data(), 4, P, fo);
+    fwrite(g0.data(), 4, C, fo);
+    if (dims == 3) fwrite(g1.data(), 4, C, fo);
+    fclose(fo);
+    return 0;
+  }
   const int S = dims == 2 ? 4 : 2;
   const size_t KK = dims == 2 ? static_cast<size_t>(K) * K : K;
   const size_t P = static_cast<size_t>(B) * C * H * W;   // 1-D: H == 1, W == N

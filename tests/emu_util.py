@@ -11,10 +11,10 @@ EMU_DIR = os.path.join(ROOT, "tests", "emu")
 BUILD_DIR = os.path.join(EMU_DIR, "_build")
 EXE = os.path.join(BUILD_DIR, "emu_driver")
 SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(ROOT, "wtconv_amd", "csrc", "mfma2d.hip"),
-           os.path.join(EMU_DIR, "emu_driver.cpp")]
+           os.path.join(ROOT, "wtconv_amd", "csrc", "block.hip"), os.path.join(EMU_DIR, "emu_driver.cpp")]
 DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
                   ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h", "kernels2d_mfma_wgrad.h",
-                   "kernels2d_stream.h", "mfma2d.h", "plan.h")] + [
+                   "kernels2d_stream.h", "mfma2d.h", "plan.h", "kernels_block.h", "wgrad_finish.h")] + [
     os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
 
 
@@ -110,3 +110,29 @@ def run(dims, x, g, base_w, base_b, base_s, wt_ws, wt_ss, K, dtype=0, pdtype=0, 
         res["dwt_ss"].append(take(s.size, s.shape))
     assert pos == raw.size
     return res
+
+
+def run_block(kind, a0, a1, p0, p1, dtype=0, pdtype=0, nhwc=1, timeout=600):
+    """The block passes on the host.  kind = "norm": a0 = x (B,C,H,W), a1 = dy ((B,H,W,C) if nhwc else (B,C,H,W)),
+    p0 = weight, p1 = bias; returns out, dx, dweight, dbias.  kind = "residual": a0 = y (B,H,W,C), a1 = shortcut
+    (B,C,H,W), p0 = gamma, p1 = dout (B,C,H,W); returns out, dy, dgamma.  float32 numpy arrays."""
+    exe = build()
+    norm = kind == "norm"
+    B, C, H, W = (a0.shape if norm else a1.shape)
+    hdr = np.array([3 if norm else 4, B, C, H, W, int(nhwc), 0, dtype, pdtype, 0], dtype=np.int32)
+    parts = [hdr.tobytes()] + [np.ascontiguousarray(a, dtype=np.float32).tobytes() for a in (a0, a1, p0, p1)]
+    with tempfile.TemporaryDirectory() as td:
+        fin, fout = os.path.join(td, "in.bin"), os.path.join(td, "out.bin")
+        with open(fin, "wb") as f:
+            f.write(b"".join(parts))
+        env = dict(os.environ)
+        env["ASAN_OPTIONS"] = "detect_leaks=0"
+        r = subprocess.run([exe, fin, fout], capture_output=True, text=True, timeout=timeout, env=env)
+        if r.returncode != 0:
+            raise RuntimeError(f"emu_driver failed ({r.returncode}):\n{r.stderr[-4000:]}")
+        raw = np.fromfile(fout, dtype=np.float32)
+    P = B * C * H * W
+    if norm:
+        oshape = (B, H, W, C) if nhwc else (B, C, H, W)
+        return raw[:P].reshape(oshape), raw[P:2 * P].reshape(B, C, H, W), raw[2 * P:2 * P + C], raw[2 * P + C:]
+    return raw[:P].reshape(B, C, H, W), raw[P:2 * P].reshape(B, H, W, C), raw[2 * P:]

@@ -27,7 +27,7 @@ def test_header_symbols_are_exported(lib):
     assert declared == set(_lib.EXPORTS), (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.wtconv_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.wtconv_abi_version() == _lib.ABI_VERSION == 5
     assert lib.wtconv_max_kernel_size() == 7
 
 

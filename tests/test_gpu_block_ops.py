@@ -63,7 +63,8 @@ def test_argument_checks(hip_device):
     with pytest.raises(RuntimeError, match="even"):
         block_ops.channel_norm(x, w, w, 1e-6, True)
     x = torch.randn(1, 4, 4, 4, device=hip_device)
-    assert not block_ops.usable(x.requires_grad_(True))       # training: nothing here is differentiable
+    assert not block_ops.usable(x.requires_grad_(True))       # recorded by autograd: the plain functions are not differentiable ...
+    assert block_ops.usable(x, training=True)                 # ... the *_fn variants are
     assert not block_ops.usable(torch.randn(1, 4, 4, 4))      # CPU tensor
     with pytest.raises(ValueError, match="does not match"):
         block_ops.block_residual(torch.randn(1, 4, 4, 3, device=hip_device), torch.randn(1, 4, 4, 4, device=hip_device), None)
@@ -95,3 +96,142 @@ def test_model_inference_fused_blocks_match_plain_blocks(hip_device, dtype, monk
         torch.testing.assert_close(fused, plain, rtol=1e-4, atol=1e-4)
     else:
         U.assert_bf16(fused, plain, "model logits")
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype,pdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_channel_norm_backward(hip_device, shape, dtype, pdtype, nhwc):
+    """dx, dweight, dbias of the backward kernel against torch autograd through F.layer_norm in float64."""
+    from wtconv_amd import block_ops
+    B, C, H, W = shape
+    gen = torch.Generator().manual_seed(B * 31 + C)
+    x = (torch.randn(shape, generator=gen) * 2 + 0.5).to(dtype)
+    w = (torch.randn(C, generator=gen) * 0.5 + 1).to(pdtype)
+    b = torch.randn(C, generator=gen).to(pdtype)
+    dy = torch.randn((B, H, W, C) if nhwc else shape, generator=gen).to(dtype)
+    xr = x.double().requires_grad_(True)
+    wr, br = w.double().requires_grad_(True), b.double().requires_grad_(True)
+    _ref_norm(xr, wr, br, 1e-6, nhwc).backward(dy.double())
+    xd = x.to(hip_device).requires_grad_(True)
+    wd, bd = w.to(hip_device).requires_grad_(True), b.to(hip_device).requires_grad_(True)
+    out = block_ops.channel_norm_fn(xd, wd, bd, 1e-6, nhwc)
+    out.backward(dy.to(hip_device))
+    torch.cuda.synchronize()
+    # dx = rstd * (g - mean(g) - xh * mean(g * xh)) cancels (for two channels almost completely: xh is +-1 there), so the
+    # absolute floor is set by the size of its terms, rstd * |dy * w|, not by the size of the result
+    xf = x.double()
+    rstd = 1.0 / torch.sqrt(xf.var(dim=1, unbiased=False, keepdim=True) + 1e-6)
+    dyn = dy.double().permute(0, 3, 1, 2) if nhwc else dy.double()
+    terms = (rstd * dyn * w.double().reshape(1, -1, 1, 1)).pow(2).mean().sqrt().item()
+    tol_x = (U.FP32_RTOL, max(U.FP32_ATOL, 1e-6 * terms)) if dtype == torch.float32 else (U.BF16_RTOL, U.BF16_RTOL * terms)
+    torch.testing.assert_close(xd.grad.double().cpu(), xr.grad, rtol=tol_x[0], atol=tol_x[1],
+                               msg=lambda m: f"dx {shape} nhwc={nhwc}: {m}")
+    # parameter gradients are fp32 sums of products of the (rounded) tensors; compared at the parameter dtype's bar
+    pcheck = U.assert_fp32 if (dtype == torch.float32 and pdtype == torch.float32) else U.assert_bf16
+    pcheck(wd.grad.float().cpu(), wr.grad.float(), f"dweight {shape}")
+    pcheck(bd.grad.float().cpu(), br.grad.float(), f"dbias {shape}")
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype,pdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16)])
+def test_block_residual_backward(hip_device, shape, dtype, pdtype):
+    """dy, dshortcut, dgamma against torch autograd through permute / mul / add in float64."""
+    from wtconv_amd import block_ops
+    B, C, H, W = shape
+    gen = torch.Generator().manual_seed(B * 13 + C)
+    y = torch.randn(B, H, W, C, generator=gen).to(dtype)
+    sc = torch.randn(shape, generator=gen).to(dtype)
+    gamma = (torch.randn(C, generator=gen) * 0.7).to(pdtype)
+    dout = torch.randn(shape, generator=gen).to(dtype)
+    yr, scr, gr = (t.double().requires_grad_(True) for t in (y, sc, gamma))
+    (yr.permute(0, 3, 1, 2) * gr.reshape(1, -1, 1, 1) + scr).backward(dout.double())
+    yd, scd, gd = (t.to(hip_device).requires_grad_(True) for t in (y, sc, gamma))
+    block_ops.block_residual_fn(yd, scd, gd).backward(dout.to(hip_device))
+    torch.cuda.synchronize()
+    check = U.assert_fp32 if dtype == torch.float32 else U.assert_bf16
+    check(yd.grad.float().cpu(), yr.grad.float(), f"dy {shape}")
+    check(scd.grad.float().cpu(), scr.grad.float(), f"dshortcut {shape}")
+    check(gd.grad.float().cpu(), gr.grad.float(), f"dgamma {shape}")
+
+
+def test_model_training_fused_blocks_match_plain_blocks(hip_device, monkeypatch):
+    """One training step of a small WTConvNeXt (fp32): loss and every parameter gradient with the fused block passes
+    (forward and backward kernels) against the same model on the plain torch passes."""
+    import wtconvnext
+    from wtconv_amd import block_ops
+    torch.manual_seed(0)
+    m = wtconvnext.WTConvNeXt(depths=(1, 1, 2, 1), dims=(16, 32, 64, 128), num_classes=10, ls_init_value=0.5).to(hip_device).train()
+    x = torch.randn(3, 3, 64, 64, device=hip_device)
+    tgt = torch.randint(0, 10, (3,), device=hip_device)
+    calls = {"n": 0}
+    real = block_ops.channel_norm_fn
+
+    def counting(*a, **k):
+        calls["n"] += 1
+        return real(*a, **k)
+    monkeypatch.setattr(block_ops, "channel_norm_fn", counting)
+
+    def step():
+        for p in m.parameters():
+            p.grad = None
+        loss = torch.nn.functional.cross_entropy(m(x), tgt)
+        loss.backward()
+        torch.cuda.synchronize()
+        return loss.item(), {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+    lf, gf = step()
+    assert calls["n"] == 5 + 4 + 1          # block norms, stem + 3 downsample norms, head norm
+    monkeypatch.setattr(block_ops, "usable", lambda *a, **k: False)
+    lp, gp = step()
+    assert abs(lf - lp) <= 1e-5 * max(abs(lp), 1.0)
+    assert set(gf) == set(gp)
+    for n in gp:
+        scale = gp[n].abs().max().item()
+        torch.testing.assert_close(gf[n], gp[n], rtol=1e-3, atol=1e-5 + 1e-4 * scale, msg=lambda s, n=n: f"{n}: {s}")
+
+
+def test_block_mlp_only_finetuning_keeps_the_mlp_gradients(hip_device):
+    """Everything frozen but the MLP of a block, input without gradient: the MLP parameters must still receive their
+    gradients (the residual pass goes through the differentiable function, not through raw pointers)."""
+    import wtconvnext
+    torch.manual_seed(0)
+    blk = wtconvnext.wtconvnext.WTConvNeXtBlock(16, wt_levels=2, ls_init_value=0.5).to(hip_device)
+    for p in blk.parameters():
+        p.requires_grad_(False)
+    for p in blk.mlp.parameters():
+        p.requires_grad_(True)
+    x = torch.randn(2, 16, 14, 14, device=hip_device)
+    blk(x).square().sum().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().sum() > 0 for p in blk.mlp.parameters())
+    ref = [p.grad.clone() for p in blk.mlp.parameters()]
+    # the same through the plain torch passes
+    from wtconv_amd import block_ops
+    real = block_ops.usable
+    block_ops.usable = lambda *a, **k: False
+    try:
+        for p in blk.mlp.parameters():
+            p.grad = None
+        blk(x).square().sum().backward()
+    finally:
+        block_ops.usable = real
+    for a, p in zip(ref, blk.mlp.parameters()):
+        torch.testing.assert_close(a, p.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_autocast_keeps_the_plain_passes(hip_device):
+    """Under torch.autocast the fused passes step aside (autocast keeps LayerNorm and the residual stream in fp32)."""
+    import wtconvnext
+    torch.manual_seed(0)
+    m = wtconvnext.WTConvNeXt(depths=(1, 1, 1, 1), dims=(16, 32, 64, 128), num_classes=10).to(hip_device).eval()
+    x = torch.randn(2, 3, 64, 64, device=hip_device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        a = m(x)
+        from wtconv_amd import block_ops
+        real = block_ops.usable
+        block_ops.usable = lambda *a_, **k: False
+        try:
+            b = m(x)
+        finally:
+            block_ops.usable = real
+    assert a.dtype == b.dtype and torch.equal(a, b)

@@ -296,3 +296,51 @@ def test_emulated_1d_fused_backward(B, C, N, K, L, bias, dtype, pdtype):
     got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K, dtype=dtype, pdtype=pdtype, fused_bwd=True)
     tol = 1e-2 if dtype else 2e-5
     _compare(got, _oracle(1, x, g, bw, bb, bs, ws, ss), rtol=tol, atol_scale=tol)
+
+
+@pytest.mark.parametrize("B,C,H,W,dtype,pdtype,nhwc", [
+    (2, 6, 5, 3, 0, 0, 1),        # odd pixel count: element-wise rows, a ragged last tile
+    (1, 10, 9, 13, 0, 0, 0),      # NCHW output (LayerNorm2d), two tiles
+    (2, 4, 1, 1, 0, 0, 1),        # a single pixel
+    (1, 96, 6, 6, 1, 1, 1),       # bf16 tensors and parameters, 4-element vector rows
+    (1, 24, 8, 10, 1, 0, 0),      # bf16 tensors (tile of floats forward), fp32 parameters
+])
+def test_emulated_channel_norm(B, C, H, W, dtype, pdtype, nhwc):
+    """wtconv_channel_norm and its backward on the host under the sanitizers, against torch in float64."""
+    rng = np.random.default_rng(B * 100 + C)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    x, w, b = f(B, C, H, W) * 2 + 0.5, f(C) * 0.5 + 1, f(C)
+    dy = f(B, H, W, C) if nhwc else f(B, C, H, W)
+    if dtype:
+        x, dy = _bf16_round(x), _bf16_round(dy)
+    if pdtype:
+        w, b = _bf16_round(w), _bf16_round(b)
+    out, dx, dw, db = emu_util.run_block("norm", x, dy, w, b, dtype, pdtype, nhwc)
+    tx, tw, tb = (torch.from_numpy(a).double().requires_grad_(True) for a in (x, w, b))
+    ref = torch.nn.functional.layer_norm(tx.permute(0, 2, 3, 1), (C,), tw, tb, 1e-6)
+    ref = ref if nhwc else ref.permute(0, 3, 1, 2)
+    ref.backward(torch.from_numpy(dy).double())
+    tol = 1e-2 if dtype else 2e-5
+    terms = float(np.sqrt(np.mean((dy.astype(np.float64) * 2.0) ** 2)))      # scale of the terms dx cancels between
+    np.testing.assert_allclose(out, ref.detach().numpy(), rtol=tol, atol=tol)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=tol, atol=tol * max(terms, 1.0))
+    np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=tol, atol=tol * max(1.0, float(np.abs(tw.grad.numpy()).max())))
+    np.testing.assert_allclose(db, tb.grad.numpy(), rtol=tol, atol=tol * max(1.0, float(np.abs(tb.grad.numpy()).max())))
+
+
+@pytest.mark.parametrize("B,C,H,W,dtype", [(2, 6, 5, 3, 0), (1, 10, 9, 13, 0), (2, 4, 1, 1, 0), (1, 96, 6, 6, 1)])
+def test_emulated_block_residual(B, C, H, W, dtype):
+    """wtconv_block_residual and its backward on the host under the sanitizers, against torch in float64."""
+    rng = np.random.default_rng(B * 7 + C)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    y, sc, gamma, dout = f(B, H, W, C), f(B, C, H, W), f(C) * 0.7, f(B, C, H, W)
+    if dtype:
+        y, sc, gamma, dout = (_bf16_round(a) for a in (y, sc, gamma, dout))
+    out, dy, dg = emu_util.run_block("residual", y, sc, gamma, dout, dtype, dtype)
+    ty, ts, tg = (torch.from_numpy(a).double().requires_grad_(True) for a in (y, sc, gamma))
+    ref = ty.permute(0, 3, 1, 2) * tg.reshape(1, -1, 1, 1) + ts
+    ref.backward(torch.from_numpy(dout).double())
+    tol = 1e-2 if dtype else 2e-5
+    np.testing.assert_allclose(out, ref.detach().numpy(), rtol=tol, atol=tol)
+    np.testing.assert_allclose(dy, ty.grad.numpy(), rtol=tol, atol=tol)
+    np.testing.assert_allclose(dg, tg.grad.numpy(), rtol=tol, atol=tol * max(1.0, float(np.abs(tg.grad.numpy()).max())))

@@ -8,7 +8,7 @@ from . import _build
 MAX_LEVELS = 5
 F32, BF16, F16 = 0, 1, 2
 PASS_FORWARD, PASS_BACKWARD_INPUT, PASS_BACKWARD_PARAMS, PASS_BACKWARD = 0, 1, 2, 3
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class Params(ctypes.Structure):
@@ -46,6 +46,9 @@ EXPORTS["wtconv1d_backward_params"] = (
 _f = ctypes.c_float
 EXPORTS["wtconv_channel_norm"] = (_i, [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _i, _p])
 EXPORTS["wtconv_block_residual"] = (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p])
+EXPORTS["wtconv_block_workspace_bytes"] = (_z, [_i, _i, _i, _i])
+EXPORTS["wtconv_channel_norm_backward"] = (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _i, _p, _z, _p])
+EXPORTS["wtconv_block_residual_backward"] = (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _z, _p])
 
 _lib = None
 _lock = threading.Lock()

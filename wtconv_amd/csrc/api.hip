@@ -131,12 +131,12 @@ static int run_plane2d_k(int K, int tj1, const void* x, void* out, const float* 
 
 template <typename T, int K, int L, typename Geo = PlaneGeoRuntime>
 static int run_wgrad2d(const void* x, const void* g, float* partial, const Plan2D& pl, int B, int bchunk,
-                       int nchunk, hipStream_t stream) {
+                       int nchunk, const FinishArgs& fin, hipStream_t stream) {
   auto kern = wt2d_wgrad_kernel<T, K, L, kTJW, Geo>;
   const size_t lds = static_cast<size_t>(pl.lds_floats) * sizeof(float);
   if (int e = allow_lds(kern, lds)) return e;
   WT_LAUNCH(kern, dim3(pl.C, nchunk), dim3(512), lds, stream, static_cast<const T*>(x), static_cast<const T*>(g),
-            partial, pl, B, bchunk);
+            partial, pl, B, bchunk, fin);
   return check_launch("wt2d_wgrad_kernel");
 }
 
@@ -144,7 +144,7 @@ static int run_wgrad2d(const void* x, const void* g, float* partial, const Plan2
 // constant.  Returns 1 if the launch is not one of them, else the launch's result.
 template <typename T>
 static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
-                              int bchunk, int nchunk, hipStream_t stream) {
+                              int bchunk, int nchunk, const FinishArgs& fin, hipStream_t stream) {
 #ifndef WT_EMULATE
   if (K != 5 || pl.H != pl.W) return 1;
 #define WT_TRY(H_, L_)                                                                                   \
@@ -153,7 +153,7 @@ static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float*
     using G = WgradGeoStatic<H_, H_, 5, L_, PB>;                                                         \
     constexpr Plan2D gp = G::plan();                                                                     \
     if (same_wgrad_geometry(gp, pl))                                                                     \
-      return run_wgrad2d<T, 5, L_, G>(x, g, partial, pl, B, bchunk, nchunk, stream);                     \
+      return run_wgrad2d<T, 5, L_, G>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);                     \
     return 1;                                                                                            \
   }
   WT_TRY(56, 3) WT_TRY(28, 3) WT_TRY(14, 2) WT_TRY(7, 2)
@@ -164,25 +164,25 @@ static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float*
 
 template <typename T, int K>
 static int run_wgrad2d_l(int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
-                         int bchunk, int nchunk, hipStream_t stream) {
+                         int bchunk, int nchunk, const FinishArgs& fin, hipStream_t stream) {
   switch (L) {
-    case 1: return run_wgrad2d<T, K, 1>(x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 2: return run_wgrad2d<T, K, 2>(x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 3: return run_wgrad2d<T, K, 3>(x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 4: return run_wgrad2d<T, K, 4>(x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 5: return run_wgrad2d<T, K, 5>(x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 1: return run_wgrad2d<T, K, 1>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 2: return run_wgrad2d<T, K, 2>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 3: return run_wgrad2d<T, K, 3>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 4: return run_wgrad2d<T, K, 4>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 5: return run_wgrad2d<T, K, 5>(x, g, partial, pl, B, bchunk, nchunk, fin, stream);
   }
   return fail(WTCONV_E_ARG, "wt_levels %d", L);
 }
 
 template <typename T>
 static int run_wgrad2d_k(int K, int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
-                         int bchunk, int nchunk, hipStream_t stream) {
+                         int bchunk, int nchunk, const FinishArgs& fin, hipStream_t stream) {
   switch (K) {
-    case 1: return run_wgrad2d_l<T, 1>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 3: return run_wgrad2d_l<T, 3>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 5: return run_wgrad2d_l<T, 5>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
-    case 7: return run_wgrad2d_l<T, 7>(L, x, g, partial, pl, B, bchunk, nchunk, stream);
+    case 1: return run_wgrad2d_l<T, 1>(L, x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 3: return run_wgrad2d_l<T, 3>(L, x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 5: return run_wgrad2d_l<T, 5>(L, x, g, partial, pl, B, bchunk, nchunk, fin, stream);
+    case 7: return run_wgrad2d_l<T, 7>(L, x, g, partial, pl, B, bchunk, nchunk, fin, stream);
   }
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
@@ -675,6 +675,26 @@ static unsigned char scratch[kStaticScratchBytes];
 static int static_scratch(const char*, void** ptr) { *ptr = scratch; return 0; }
 #endif
 
+static int check_grad_table(const char* fn, const wtconv_params* params, const wtconv_param_grads* grads, int L) {
+  if (grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
+  if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
+      (params->base_bias != nullptr && grads->base_bias == nullptr))
+    return fail(WTCONV_E_ARG, "%s: null gradient pointer", fn);
+  for (int l = 0; l < L; ++l)
+    if (grads->wt_weight[l] == nullptr || grads->wt_scale[l] == nullptr)
+      return fail(WTCONV_E_ARG, "%s: null gradient pointer at level %d", fn, l);
+  return 0;
+}
+
+static GradTable to_grad_table(const wtconv_param_grads* grads, int L) {
+  GradTable gt = {};
+  gt.base_weight = grads->base_weight;
+  gt.base_bias = grads->base_bias;
+  gt.base_scale = grads->base_scale;
+  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
+  return gt;
+}
+
 }  // namespace wt
 
 using namespace wt;
@@ -710,6 +730,7 @@ size_t wtconv2d_workspace_bytes(int B, int C, int H, int W, int K, int levels, i
                2 * make_stream2d(B, C, H, W, levels).floats;
     }
     if (mfloats > floats) floats = mfloats;
+    floats = round_up64(floats) + static_cast<size_t>(C);      // one ticket word per channel behind the records
   } else {
     // the dtype is not an argument here: size for the larger of the two (fp32 tensors take
     // three split tables) whenever either could run on the matrix-core kernels
@@ -785,19 +806,31 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   float* partial = static_cast<float*>(workspace);
   int e;
   const Mfma2dWgradQuery mq = mfma2d_wgrad_query(B, C, H, W, K, L, dtype);
+  const bool resident = mq.ok || wgrad_fits_lds(B, C, H, W, K, L);
+  // The plane-resident first-stage kernels finish their channels themselves (last workgroup of a channel): one ticket
+  // word per channel at the end of the workspace, cleared by a small launch of its own.
+  FinishArgs fin = {};
+  if (resident) {
+    fin.tickets = reinterpret_cast<unsigned*>(static_cast<char*>(workspace) + need) - C;
+    fin.prm = to_table(params, L);
+    fin.pdtype = param_dtype;
+    fin.gt = to_grad_table(grads, L);
+    WT_LAUNCH(zero_tickets_kernel, dim3((C + 255) / 256), dim3(256), 0, stream, fin.tickets, C);
+    if (int ze = check_launch("zero_tickets_kernel")) return ze;
+  }
   if (mq.ok) {
     nchunk = mq.nchunk;
-    e = mfma2d_wgrad_pass(fn, x, grad_out, partial, B, C, H, W, K, L, stream);
-  } else if (wgrad_fits_lds(B, C, H, W, K, L)) {
+    e = mfma2d_wgrad_pass(fn, x, grad_out, partial, B, C, H, W, K, L, fin, stream);
+  } else if (resident) {
     const int pb = wgrad_planes_per_iter(B, H, W, K, L);
     Plan2D pl = make_plan2d(B, C, H, W, K, L, true, 512, esz, x, grad_out, nullptr, pb);
     finish_wgrad_plan(&pl, K);
     wgrad_chunks(B, C, pb, kWgradResident, &bchunk, &nchunk);
-    e = dtype == WTCONV_F32   ? run_wgrad2d_static<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
-        : dtype == WTCONV_F16 ? run_wgrad2d_static<f16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream)
+    e = dtype == WTCONV_F32   ? run_wgrad2d_static<float>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, fin, stream)
+        : dtype == WTCONV_F16 ? run_wgrad2d_static<f16_t>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, fin, stream)
                               : 1;
     if (e == 1)
-      e = WT_BY_DTYPE(dtype, run_wgrad2d_k<T_>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, stream));
+      e = WT_BY_DTYPE(dtype, run_wgrad2d_k<T_>(K, L, x, grad_out, partial, pl, B, bchunk, nchunk, fin, stream));
   } else {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     nchunk = stream_chunks(B, C, H, W);
@@ -806,12 +839,8 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
     float* pyr_g = pyr_x + sp.floats;
     e = WT_BY_DTYPE(dtype, run_stream2d_wgrad_k<T_>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream));
   }
-  if (e) return e;
-  GradTable gt = {};
-  gt.base_weight = grads->base_weight;
-  gt.base_bias = grads->base_bias;
-  gt.base_scale = grads->base_scale;
-  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
+  if (e || resident) return e;
+  const GradTable gt = to_grad_table(grads, L);
   const int nrec = (1 + 4 * L) * K * K + 1;
   WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(finish_threads(nrec)), static_cast<size_t>(nrec) * sizeof(float),
             stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 4, L, K * K);
@@ -917,26 +946,6 @@ int wtconv1d_backward_params(const void* x, const void* grad_out, const wtconv_p
   WT_LAUNCH(wgrad_finish_kernel, dim3(C), dim3(finish_threads(nrec)), static_cast<size_t>(nrec) * sizeof(float),
             stream, partial, nchunk, to_table(params, L), param_dtype, gt, C, 2, L, K);
   return check_launch("wgrad_finish_kernel");
-}
-
-static int check_grad_table(const char* fn, const wtconv_params* params, const wtconv_param_grads* grads, int L) {
-  if (grads == nullptr) return fail(WTCONV_E_ARG, "%s: null tensor pointer", fn);
-  if (grads->base_weight == nullptr || grads->base_scale == nullptr ||
-      (params->base_bias != nullptr && grads->base_bias == nullptr))
-    return fail(WTCONV_E_ARG, "%s: null gradient pointer", fn);
-  for (int l = 0; l < L; ++l)
-    if (grads->wt_weight[l] == nullptr || grads->wt_scale[l] == nullptr)
-      return fail(WTCONV_E_ARG, "%s: null gradient pointer at level %d", fn, l);
-  return 0;
-}
-
-static GradTable to_grad_table(const wtconv_param_grads* grads, int L) {
-  GradTable gt = {};
-  gt.base_weight = grads->base_weight;
-  gt.base_bias = grads->base_bias;
-  gt.base_scale = grads->base_scale;
-  for (int l = 0; l < L; ++l) { gt.wt_weight[l] = grads->wt_weight[l]; gt.wt_scale[l] = grads->wt_scale[l]; }
-  return gt;
 }
 
 int wtconv1d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,

@@ -14,15 +14,17 @@ namespace {
 // Largest power-of-two pixel tile (8..64) whose [C][tp + 1] elements of `esz` bytes, plus the per-pixel statistics,
 // stay within 48 KB of LDS (three workgroups per CU); false if even 8 pixels do not fit or the sizes overflow the
 // indexing.
-bool make_block_tile(int C, int HW, size_t esz, BlockTile* out, size_t* lds_bytes) {
+// `ntile` tiles per workgroup: one in the forward kernels, two in the backward ones (budget 64 KB there).
+bool make_block_tile(int C, int HW, size_t esz, int ntile, BlockTile* out, size_t* lds_bytes) {
   BlockTile t = {};
   t.C = C; t.HW = HW;
   int tp = 64;
-  // tile (rounded up to 16 bytes), then floats: two sets of partial sums [256 / p][p], mean and rstd [2][p],
+  // tiles (rounded up to 16 bytes), then floats: two sets of partial sums [256 / p][p], per-pixel statistics [4][p],
   // weight and bias [2][C]
-  auto tile_bytes = [&](int p) { return (static_cast<size_t>(C) * (p + 1) * esz + 15) / 16 * 16; };
-  auto bytes = [&](int p) { return tile_bytes(p) + (2 * kBlockThreads + 2 * p + 2 * static_cast<size_t>(C)) * sizeof(float); };
-  while (tp > 8 && bytes(tp) > 48 * 1024) tp >>= 1;
+  auto tile_bytes = [&](int p) { return (static_cast<size_t>(ntile) * C * (p + 1) * esz + 15) / 16 * 16; };
+  auto bytes = [&](int p) { return tile_bytes(p) + (2 * kBlockThreads + 4 * p + 2 * static_cast<size_t>(C)) * sizeof(float); };
+  const size_t budget = ntile == 1 ? 48 * 1024 : 64 * 1024;
+  while (tp > 8 && bytes(tp) > budget) tp >>= 1;
   if (bytes(tp) > kLdsLimitBytes) return false;
   while (tp > 8 && tp / 2 >= HW) tp >>= 1;          // tiny images: no lanes without a pixel
   t.tp = tp;
@@ -42,24 +44,24 @@ bool make_block_tile(int C, int HW, size_t esz, BlockTile* out, size_t* lds_byte
 }
 
 struct TileKey {
-  int C, HW, esz;
+  int C, HW, esz;      // esz: bytes of a tile element, negated for the two-tile plans of the backward kernels
   bool operator==(const TileKey& o) const { return C == o.C && HW == o.HW && esz == o.esz; }
 };
 struct TileKeyHash {
   size_t operator()(const TileKey& k) const {
-    return (static_cast<size_t>(k.C) << 32) ^ (static_cast<size_t>(k.HW) << 3) ^ static_cast<size_t>(k.esz);
+    return (static_cast<size_t>(k.C) << 32) ^ (static_cast<size_t>(k.HW) << 4) ^ static_cast<size_t>(k.esz + 8);
   }
 };
 struct TileVal { bool ok; BlockTile t; size_t lds; int esz; };      // esz: bytes of a tile element
 
-const TileVal& block_tile_cached(int C, int HW, int esz) {
+const TileVal& block_tile_cached(int C, int HW, int esz, int ntile = 1) {
   static thread_local std::unordered_map<TileKey, TileVal, TileKeyHash> cache;
-  const TileKey key = {C, HW, esz};
+  const TileKey key = {C, HW, ntile == 1 ? esz : -esz};
   auto it = cache.find(key);
   if (it == cache.end()) {
     if (cache.size() > 4096) cache.clear();
     TileVal v = {};
-    v.ok = make_block_tile(C, HW, static_cast<size_t>(esz), &v.t, &v.lds);
+    v.ok = make_block_tile(C, HW, static_cast<size_t>(esz), ntile, &v.t, &v.lds);
     v.esz = esz;
     it = cache.emplace(key, v).first;
   }
@@ -68,15 +70,15 @@ const TileVal& block_tile_cached(int C, int HW, int esz) {
 
 // float_tile: the caller can keep bf16 tensors as floats in LDS; taken where that still gives 64 pixels per tile.
 int check_block_args(const char* fn, int B, int C, int HW, int dtype, int pdtype, const TileVal** tv,
-                     bool float_tile = false) {
+                     bool float_tile = false, int ntile = 1) {
   if (B <= 0 || C <= 0 || HW <= 0) return fail(WTCONV_E_ARG, "%s: sizes must be positive (got B=%d C=%d HW=%d)", fn, B, C, HW);
   if (C % 2) return fail(WTCONV_E_UNSUPPORTED, "%s: the channel count must be even (got %d)", fn, C);
   if ((dtype != WTCONV_F32 && dtype != WTCONV_BF16) || (pdtype != WTCONV_F32 && pdtype != WTCONV_BF16))
     return fail(WTCONV_E_ARG, "%s: unknown dtype code", fn);
   if (B > 65535) return fail(WTCONV_E_UNSUPPORTED, "%s: batch %d exceeds the launch grid", fn, B);
   if (static_cast<long long>(C) * HW > 0x7fffffffLL) return fail(WTCONV_E_UNSUPPORTED, "%s: an image of %d x %d elements is too large", fn, C, HW);
-  const TileVal* vp = &block_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2);
-  if (float_tile && dtype != WTCONV_F32) {
+  const TileVal* vp = &block_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2, ntile);
+  if (ntile == 1 && float_tile && dtype != WTCONV_F32) {
     const TileVal& vf = block_tile_cached(C, HW, 4);
     if (vf.ok && vf.t.tp == 64) vp = &vf;
   }
@@ -149,4 +151,99 @@ extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const 
                : launch(block_residual_kernel<float, false>, static_cast<float*>(nullptr));
   return vec ? launch(block_residual_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
              : launch(block_residual_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+}
+
+// ---- backward passes ---------------------------------------------------------------------------------------
+
+// Floats of workspace: one record per workgroup (B * tiles of them) of 2 C floats (the norm's dweight and dbias; the
+// residual's dgamma takes the first C of each).
+extern "C" size_t wtconv_block_workspace_bytes(int B, int C, int HW, int dtype) {
+  if (B <= 0 || C <= 0 || HW <= 0 || (dtype != WTCONV_F32 && dtype != WTCONV_BF16)) return 0;
+  const TileVal& v = block_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2, 2);
+  if (!v.ok) return 0;
+  const size_t bytes = static_cast<size_t>(B) * v.t.tiles * 2 * C * sizeof(float);
+  return (bytes + 255) / 256 * 256;
+}
+
+static int launch_column_sum(const float* partial, int nrec, int ncol, float* out0, float* out1, int split,
+                             hipStream_t stream) {
+  WT_LAUNCH(column_sum_kernel, dim3((ncol + 63) / 64), dim3(kBlockThreads), 0, stream, partial, nrec, ncol, out0, out1,
+            split);
+  return check_launch("column_sum_kernel");
+}
+
+extern "C" int wtconv_channel_norm_backward(const void* x, const void* dy, const void* weight, void* dx, float* dweight,
+                                            float* dbias, int B, int C, int HW, float eps, int dtype, int param_dtype,
+                                            int dy_nhwc, void* workspace, size_t workspace_bytes, void* stream_) {
+  const char* fn = "wtconv_channel_norm_backward";
+  const TileVal* tv = nullptr;
+  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv, false, 2)) return e;
+  if (x == nullptr || dy == nullptr || weight == nullptr || dx == nullptr || dweight == nullptr || dbias == nullptr)
+    return fail(WTCONV_E_ARG, "%s: null pointer", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) % esz) || (reinterpret_cast<uintptr_t>(dx) % (2 * esz)) ||
+      (reinterpret_cast<uintptr_t>(dy) % (2 * esz)))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned (x to one element, dy and dx to two)", fn);
+  const size_t need = wtconv_block_workspace_bytes(B, C, HW, dtype);
+  if (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) % 4))
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const dim3 grid(tv->t.tiles, B);
+  const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0 &&
+                   reinterpret_cast<uintptr_t>(dx) % (4 * esz) == 0 &&
+                   (dy_nhwc || reinterpret_cast<uintptr_t>(dy) % (4 * esz) == 0);
+  float* partial = static_cast<float*>(workspace);
+  auto launch = [&](auto kern, auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (int e = allow_lds(kern, tv->lds)) return e;
+    WT_LAUNCH(kern, grid, dim3(kBlockThreads), tv->lds, stream, static_cast<const T*>(x), static_cast<const T*>(dy),
+              weight, param_dtype, eps, dy_nhwc, static_cast<T*>(dx), partial, tv->t);
+    return check_launch("channel_norm_bwd_kernel");
+  };
+  int e;
+  if (dtype == WTCONV_F32)
+    e = vec ? launch(channel_norm_bwd_kernel<float, true>, static_cast<float*>(nullptr))
+            : launch(channel_norm_bwd_kernel<float, false>, static_cast<float*>(nullptr));
+  else
+    e = vec ? launch(channel_norm_bwd_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
+            : launch(channel_norm_bwd_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+  if (e) return e;
+  return launch_column_sum(partial, B * tv->t.tiles, 2 * C, dweight, dbias, C, stream);
+}
+
+extern "C" int wtconv_block_residual_backward(const void* dout, const void* y, const void* gamma, void* dy, float* dgamma,
+                                              int B, int C, int HW, int dtype, int param_dtype, void* workspace,
+                                              size_t workspace_bytes, void* stream_) {
+  const char* fn = "wtconv_block_residual_backward";
+  const TileVal* tv = nullptr;
+  if (int e = check_block_args(fn, B, C, HW, dtype, param_dtype, &tv, false, 2)) return e;
+  if (dout == nullptr || y == nullptr || gamma == nullptr || dy == nullptr || dgamma == nullptr)
+    return fail(WTCONV_E_ARG, "%s: null pointer", fn);
+  const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(dout) % esz) || (reinterpret_cast<uintptr_t>(y) % (2 * esz)) ||
+      (reinterpret_cast<uintptr_t>(dy) % (2 * esz)))
+    return fail(WTCONV_E_ARG, "%s: tensor pointer not aligned (dout to one element, the NHWC tensors to two)", fn);
+  const size_t need = wtconv_block_workspace_bytes(B, C, HW, dtype);
+  if (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) % 4))
+    return fail(WTCONV_E_WORKSPACE, "%s: workspace of %zu B needed, %zu given", fn, need, workspace_bytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const dim3 grid(tv->t.tiles, B);
+  const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(dout) % (4 * esz) == 0;
+  float* partial = static_cast<float*>(workspace);
+  auto launch = [&](auto kern, auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    if (int e = allow_lds(kern, tv->lds)) return e;
+    WT_LAUNCH(kern, grid, dim3(kBlockThreads), tv->lds, stream, static_cast<const T*>(dout), static_cast<const T*>(y),
+              gamma, param_dtype, static_cast<T*>(dy), partial, tv->t);
+    return check_launch("block_residual_bwd_kernel");
+  };
+  int e;
+  if (dtype == WTCONV_F32)
+    e = vec ? launch(block_residual_bwd_kernel<float, true>, static_cast<float*>(nullptr))
+            : launch(block_residual_bwd_kernel<float, false>, static_cast<float*>(nullptr));
+  else
+    e = vec ? launch(block_residual_bwd_kernel<bf16_t, true>, static_cast<bf16_t*>(nullptr))
+            : launch(block_residual_bwd_kernel<bf16_t, false>, static_cast<bf16_t*>(nullptr));
+  if (e) return e;
+  return launch_column_sum(partial, B * tv->t.tiles, C, dgamma, dgamma, C, stream);
 }

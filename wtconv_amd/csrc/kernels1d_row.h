@@ -26,7 +26,7 @@
 
 #include "common.h"
 #include "kernels1d.h"
-#include "kernels2d.h"      // wgrad_finish_channel
+#include "wgrad_finish.h"
 
 namespace wt {
 

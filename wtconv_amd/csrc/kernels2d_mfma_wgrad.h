@@ -28,6 +28,7 @@
 
 #include "common.h"
 #include "kernels2d_mfma.h"
+#include "wgrad_finish.h"
 
 namespace wt {
 
@@ -180,7 +181,7 @@ __device__ __forceinline__ void corr_mma(const CorrTile<NX>& t, Acc (&d)[5]) {
 template <int L, int NW, bool VEC, typename Geo>
 __global__ void __launch_bounds__(NW * 64, 2)
 wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ g, float* __restrict__ partial,
-                       const WPlan plarg, int K, int bchunk) {
+                       const WPlan plarg, int K, int bchunk, const FinishArgs fin) {
   const WPlan pl = [&]() {
     if constexpr (Geo::kStatic) {
       constexpr WPlan gp = Geo::plan();
@@ -501,7 +502,8 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     if (i == 25 * (1 + 4 * L)) {
 #pragma unroll
       for (int wv = 0; wv < NW; ++wv) v += lds_ld<float>(lds, NW * kWaveBand + wv * 4);
-      rec[nrec - 1] = v;
+      if (fin.tickets != nullptr) store_shared_f32(rec + nrec - 1, v);
+      else rec[nrec - 1] = v;
       continue;
     }
     const int f = i / 25, tap = i - 25 * f;          // f = 0: base conv; else 1 + 4 (l - 1) + s
@@ -519,8 +521,12 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     float sc = 1.f;
     for (int k = 0; k < l; ++k) sc *= 0.25f;        // both pyramids were left unnormalised: 2^l each
     const int t = tap_of_frame(kh, kw, K);
-    if (t >= 0) rec[f * KK + t] = v * sc;
+    if (t >= 0) {
+      if (fin.tickets != nullptr) store_shared_f32(rec + f * KK + t, v * sc);
+      else rec[f * KK + t] = v * sc;
+    }
   }
+  wgrad_finish_if_last(fin, partial, static_cast<int>(gridDim.y), C, c, 4, L, KK, reinterpret_cast<float*>(lds));
 }
 
 }  // namespace wt

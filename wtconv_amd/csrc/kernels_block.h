@@ -40,7 +40,9 @@ __device__ __forceinline__ int div_c(int v, unsigned magic) {
 template <typename T>
 __device__ __forceinline__ void store_pair(T* p, float a, float b);
 template <> __device__ __forceinline__ void store_pair<float>(float* p, float a, float b) {
-  *reinterpret_cast<float2*>(p) = make_float2(a, b);
+  float2 v;
+  v.x = a; v.y = b;
+  *reinterpret_cast<float2*>(p) = v;
 }
 template <> __device__ __forceinline__ void store_pair<bf16_t>(bf16_t* p, float a, float b) {
   *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(a, b);
@@ -261,6 +263,195 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
         out[o] = from_f32<T>(to_f32<T>(shortcut[o]) + g * to_f32<T>(lds[c * pitch + p]));
       }
     }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ backward passes
+// The same two passes under autograd (training keeps the block's structure, wtconvnext/wtconvnext.py:125-140 of the
+// reference): tiles as above, two of them per workgroup (the saved input and the incoming gradient), in the tensors'
+// own element type.  Parameter gradients are per-workgroup partial sums in the caller's workspace -- record
+// (b * tiles + tile) holds NV vectors of C floats -- summed in record order by column_sum_kernel: two fixed stages,
+// no atomics.
+
+// LDS [C][tp + 1] -> NCHW rows (pixels past the image are dropped)
+template <typename T, bool VEC>
+__device__ __forceinline__ void tile_to_nchw(const T* lds, T* __restrict__ img, const BlockTile& t, int p0, int np, int tid) {
+  const int pitch = t.tp + 1;
+  if constexpr (VEC) {
+    const int gshift = t.tp_shift - 2;
+    const int g = tid & ((1 << gshift) - 1), c0 = tid >> gshift, cstep = kBlockThreads >> gshift;
+    const int p = 4 * g;
+    if (p < np)
+      for (int c = c0; c < t.C; c += cstep) {
+        const T* row = lds + c * pitch + p;
+        T* o = img + static_cast<size_t>(c) * t.HW + p0 + p;
+        store_pair<T>(o, to_f32<T>(row[0]), to_f32<T>(row[1]));
+        store_pair<T>(o + 2, to_f32<T>(row[2]), to_f32<T>(row[3]));
+      }
+  } else {
+    const int p = tid & (t.tp - 1), c0 = tid >> t.tp_shift, cstep = kBlockThreads >> t.tp_shift;
+    if (p < np)
+      for (int c = c0; c < t.C; c += cstep) img[static_cast<size_t>(c) * t.HW + p0 + p] = lds[c * pitch + p];
+  }
+}
+
+// NHWC tile (one contiguous run of np * C elements, C even) -> LDS [C][tp + 1]
+template <typename T>
+__device__ __forceinline__ void tile_from_nhwc(const T* __restrict__ src, T* lds, const BlockTile& t, int np, int tid) {
+  const int pitch = t.tp + 1, C = t.C;
+  const int npair = (np * C) >> 1;
+  for (int i = tid; i < npair; i += kBlockThreads) {
+    const int e = 2 * i;
+    const int pp = div_c(e, t.mg_c), c = e - pp * C;
+    T a, bb;
+    load_pair_raw<T>(src + e, a, bb);
+    lds[c * pitch + pp] = a;
+    lds[(c + 1) * pitch + pp] = bb;
+  }
+}
+
+// Backward of channel_norm_kernel.  Grid (tiles, B).  x (B, C, HW) is the forward input, dy the gradient of the
+// forward output ((B, HW, C) if dy_nhwc else (B, C, HW)), dx (B, C, HW).  Per pixel, with xh = (x - mean) * rstd and
+// g = dy * weight:  dx = rstd * (g - mean_c(g) - xh * mean_c(g * xh)).  Per channel: dweight = sum dy * xh,
+// dbias = sum dy, left as this workgroup's record {dweight[C], dbias[C]} in `partial`.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlockThreads)
+channel_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy, const void* __restrict__ weight, int pdtype,
+                        float eps, int dy_nhwc, T* __restrict__ dx, float* __restrict__ partial, const BlockTile t) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x;
+  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  const int pitch = t.tp + 1, C = t.C;
+  const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
+  T* xt = reinterpret_cast<T*>(ldsf);            // tile of x, later of dx
+  T* gt = xt + C * pitch;                        // tile of dy
+  float* psum = ldsf + t.aux;                    // [parts][tp] partial sums (two sets)
+  float* pvar = psum + kBlockThreads;
+  float* stat = pvar + kBlockThreads;            // mean[tp], rstd[tp], then the two means of the gradient terms
+  float* wgt = stat + 4 * t.tp;                  // weight[C]
+  const T* ximg = x + static_cast<size_t>(b) * C * t.HW;
+  tile_from_nchw<T, T, VEC>(ximg, xt, t, p0, tid);
+  if (dy_nhwc) tile_from_nhwc<T>(dy + (static_cast<size_t>(b) * t.HW + p0) * C, gt, t, np, tid);
+  else tile_from_nchw<T, T, VEC>(dy + static_cast<size_t>(b) * C * t.HW, gt, t, p0, tid);
+  for (int c = tid; c < C; c += kBlockThreads) wgt[c] = load_param(weight, pdtype, c);
+  __syncthreads();
+  const int p = tid & (t.tp - 1), part_i = tid >> t.tp_shift, parts = kBlockThreads >> t.tp_shift;
+  const bool live = p < np;
+  const float invC = 1.f / static_cast<float>(C);
+  float s = 0.f;
+  if (live)
+    for (int c = part_i; c < C; c += parts) s += to_f32<T>(xt[c * pitch + p]);
+  psum[part_i * t.tp + p] = s;
+  __syncthreads();
+  float mean = 0.f;
+  for (int k = 0; k < parts; ++k) mean += psum[k * t.tp + p];
+  mean *= invC;
+  float v = 0.f;
+  if (live)
+    for (int c = part_i; c < C; c += parts) {
+      const float d = to_f32<T>(xt[c * pitch + p]) - mean;
+      v += d * d;
+    }
+  pvar[part_i * t.tp + p] = v;
+  __syncthreads();
+  float var = 0.f;
+  for (int k = 0; k < parts; ++k) var += pvar[k * t.tp + p];
+  const float rstd = 1.f / sqrtf(var * invC + eps);
+  __syncthreads();                               // psum / pvar are reused below
+  float s1 = 0.f, s2 = 0.f;
+  if (live)
+    for (int c = part_i; c < C; c += parts) {
+      const float g = to_f32<T>(gt[c * pitch + p]) * wgt[c];
+      const float xh = (to_f32<T>(xt[c * pitch + p]) - mean) * rstd;
+      s1 += g;
+      s2 = fmaf(g, xh, s2);
+    }
+  psum[part_i * t.tp + p] = s1;
+  pvar[part_i * t.tp + p] = s2;
+  if (part_i == 0) { stat[p] = mean; stat[t.tp + p] = rstd; }
+  __syncthreads();
+  float m1 = 0.f, m2 = 0.f;
+  for (int k = 0; k < parts; ++k) { m1 += psum[k * t.tp + p]; m2 += pvar[k * t.tp + p]; }
+  m1 *= invC; m2 *= invC;
+  // per-channel sums over the tile's pixels (before x's tile is overwritten with dx)
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * 2 * C;
+  for (int c = tid; c < C; c += kBlockThreads) {
+    float dw = 0.f, db = 0.f;
+    for (int pp = 0; pp < np; ++pp) {
+      const float d = to_f32<T>(gt[c * pitch + pp]);
+      const float xh = (to_f32<T>(xt[c * pitch + pp]) - stat[pp]) * stat[t.tp + pp];
+      dw = fmaf(d, xh, dw);
+      db += d;
+    }
+    rec[c] = dw;
+    rec[C + c] = db;
+  }
+  __syncthreads();
+  if (live)
+    for (int c = part_i; c < C; c += parts) {
+      const float g = to_f32<T>(gt[c * pitch + p]) * wgt[c];
+      const float xh = (to_f32<T>(xt[c * pitch + p]) - mean) * rstd;
+      xt[c * pitch + p] = from_f32<T>(rstd * (g - m1 - xh * m2));
+    }
+  __syncthreads();
+  tile_to_nchw<T, VEC>(xt, dx + static_cast<size_t>(b) * C * t.HW, t, p0, np, tid);
+}
+
+// Backward of block_residual_kernel with a layer scale.  Grid (tiles, B).  dout (B, C, HW) is the gradient of the
+// block's output (the shortcut's gradient is dout itself), y (B, HW, C) the forward's NHWC input; dy (B, HW, C) =
+// gamma[c] * dout; this workgroup's record in `partial` = dgamma[C] = sum over its pixels of dout * y.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(kBlockThreads)
+block_residual_bwd_kernel(const T* __restrict__ dout, const T* __restrict__ y, const void* __restrict__ gamma, int pdtype,
+                          T* __restrict__ dy, float* __restrict__ partial, const BlockTile t) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x;
+  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  const int pitch = t.tp + 1, C = t.C;
+  const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
+  T* dt = reinterpret_cast<T*>(ldsf);            // tile of dout
+  T* yt = dt + C * pitch;                        // tile of y
+  float* wgt = ldsf + t.aux;                     // gamma[C]
+  tile_from_nchw<T, T, VEC>(dout + static_cast<size_t>(b) * C * t.HW, dt, t, p0, tid);
+  const size_t run = (static_cast<size_t>(b) * t.HW + p0) * C;
+  tile_from_nhwc<T>(y + run, yt, t, np, tid);
+  for (int c = tid; c < C; c += kBlockThreads) wgt[c] = load_param(gamma, pdtype, c);
+  __syncthreads();
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * C;
+  for (int c = tid; c < C; c += kBlockThreads) {
+    float dg = 0.f;
+    for (int pp = 0; pp < np; ++pp) dg = fmaf(to_f32<T>(dt[c * pitch + pp]), to_f32<T>(yt[c * pitch + pp]), dg);
+    rec[c] = dg;
+  }
+  T* dst = dy + run;
+  const int npair = (np * C) >> 1;
+  for (int i = tid; i < npair; i += kBlockThreads) {
+    const int e = 2 * i;
+    const int pp = div_c(e, t.mg_c), c = e - pp * C;
+    store_pair<T>(dst + e, wgt[c] * to_f32<T>(dt[c * pitch + pp]), wgt[c + 1] * to_f32<T>(dt[(c + 1) * pitch + pp]));
+  }
+}
+
+// out[v] = sum over the `nrec` records of partial[r][v], v < ncol, added in record order (grid = ceil(ncol / 64)
+// workgroups of 256 threads: four row groups per column, joined through LDS in a fixed order).
+__global__ void __launch_bounds__(kBlockThreads) column_sum_kernel(const float* __restrict__ partial, int nrec, int ncol,
+                                                                   float* __restrict__ out0, float* __restrict__ out1,
+                                                                   int split) {
+  __shared__ float red[kBlockThreads];
+  const int col = blockIdx.x * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
+  float s = 0.f;
+  if (col < ncol) {
+    const int per = (nrec + 3) / 4;
+    const int r0 = grp * per, r1 = r0 + per < nrec ? r0 + per : nrec;
+#pragma unroll 4
+    for (int r = r0; r < r1; ++r) s += partial[static_cast<size_t>(r) * ncol + col];
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  if (grp == 0 && col < ncol) {
+    const float v = (red[threadIdx.x] + red[threadIdx.x + 64]) + (red[threadIdx.x + 128] + red[threadIdx.x + 192]);
+    if (col < split) out0[col] = v;
+    else out1[col - split] = v;
   }
 }
 

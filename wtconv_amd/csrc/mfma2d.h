@@ -4,6 +4,7 @@
 #include <stddef.h>
 
 #include "common.h"
+#include "wgrad_finish.h"
 
 namespace wt {
 
@@ -21,7 +22,7 @@ int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* p
                 int K, int L, int dtype, int pdtype, hipStream_t stream, int flip);
 
 // Parameter gradients of bf16 tensors: whether the shape runs on the MFMA kernel, and the size of the
-// per-chunk partial sums it leaves in the workspace for wgrad_finish_kernel (`nchunk` records per channel).
+// per-chunk partial sums it leaves in the workspace (`nchunk` records per channel).
 struct Mfma2dWgradQuery {
   bool ok;
   int nchunk;
@@ -29,7 +30,8 @@ struct Mfma2dWgradQuery {
 };
 Mfma2dWgradQuery mfma2d_wgrad_query(int B, int C, int H, int W, int K, int L, int dtype);
 
+// `fin`: with tickets set, the kernel finishes the channels itself (no wgrad_finish_kernel launch after it).
 int mfma2d_wgrad_pass(const char* fn, const void* x, const void* grad_out, float* partial, int B, int C, int H, int W,
-                      int K, int L, hipStream_t stream);
+                      int K, int L, const FinishArgs& fin, hipStream_t stream);
 
 }  // namespace wt

@@ -271,7 +271,7 @@ const WVal& wplan_cached(int B, int C, int H, int W, int L) {
   return it->second;
 }
 
-struct WgradArgs { const void* x; const void* g; float* partial; int K, bchunk, nchunk; };
+struct WgradArgs { const void* x; const void* g; float* partial; int K, bchunk, nchunk; FinishArgs fin; };
 
 template <int L, int NW, bool VEC, typename Geo>
 int launch_wgrad(const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
@@ -279,7 +279,7 @@ int launch_wgrad(const WgradArgs& a, const WPlan& pl, hipStream_t stream) {
   const size_t lds = static_cast<size_t>(pl.lds_bytes);
   if (int e = allow_lds(kern, lds)) return e;
   WT_LAUNCH(kern, dim3(pl.C, a.nchunk), dim3(NW * 64), lds, stream, static_cast<const bf16_t*>(a.x),
-            static_cast<const bf16_t*>(a.g), a.partial, pl, a.K, a.bchunk);
+            static_cast<const bf16_t*>(a.g), a.partial, pl, a.K, a.bchunk, a.fin);
   return check_launch("wt2d_mfma_wgrad_kernel");
 }
 
@@ -314,13 +314,13 @@ Mfma2dWgradQuery mfma2d_wgrad_query(int B, int C, int H, int W, int K, int L, in
 }
 
 int mfma2d_wgrad_pass(const char* fn, const void* x, const void* grad_out, float* partial, int B, int C, int H, int W,
-                      int K, int L, hipStream_t stream) {
+                      int K, int L, const FinishArgs& fin, hipStream_t stream) {
   const WVal& v = wplan_cached(B, C, H, W, L);
   if (!v.ok) return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
   WPlan pl = v.pl;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(grad_out)) & 7u) == 0;
   const bool vec = (W % 4 == 0) && aligned;
-  const WgradArgs a = {x, grad_out, partial, K, v.bchunk, v.nchunk};
+  const WgradArgs a = {x, grad_out, partial, K, v.bchunk, v.nchunk, fin};
   switch (L) {
     case 1: return launch_wgrad_l<1>(v.nw, v.compact != 0, vec, a, pl, stream);
     case 2: return launch_wgrad_l<2>(v.nw, v.compact != 0, vec, a, pl, stream);

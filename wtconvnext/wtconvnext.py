@@ -38,8 +38,11 @@ class LayerNorm2d(nn.LayerNorm):
 
     def forward(self, x):
         ops = _block_ops()
-        if ops is not None and self.elementwise_affine and self.bias is not None and ops.usable(x, self.weight, self.bias):
-            return ops.channel_norm(x, self.weight, self.bias, self.eps, nhwc=False)      # inference: one kernel
+        if (ops is not None and self.elementwise_affine and self.bias is not None and x.is_contiguous()
+                and ops.usable(x, self.weight, self.bias, training=True)):
+            if ops.records(x, self.weight, self.bias):      # one kernel each way
+                return ops.channel_norm_fn(x, self.weight, self.bias, self.eps, False)
+            return ops.channel_norm(x, self.weight, self.bias, self.eps, nhwc=False)
         x = x.permute(0, 2, 3, 1)
         x = F.layer_norm(x, self.normalized_shape, self.weight, self.bias, self.eps)
         return x.permute(0, 3, 1, 2)
@@ -91,16 +94,24 @@ class WTConvNeXtBlock(nn.Module):
         ops = _block_ops()
         drops = self.training and not isinstance(self.drop_path, nn.Identity)
         if (ops is not None and not drops and x.is_contiguous() and shortcut.is_contiguous()
-                and ops.usable(x, self.norm.weight, self.norm.bias, self.gamma)
-                and ops.usable(shortcut)):
-            # inference on the GPU: NCHW -> LayerNorm -> NHWC, and NHWC -> layer scale -> + shortcut -> NCHW, are one
-            # kernel each instead of a layout copy plus an elementwise pass each
-            y = self.mlp(ops.channel_norm(x, self.norm.weight, self.norm.bias, self.norm.eps, nhwc=True))
-            # the MLP may still record for autograd (its own parameters can be trainable while everything before it
-            # is frozen) or change the dtype; the residual kernel takes raw pointers, so only a plain tensor of the
-            # shortcut's type goes there
+                and ops.usable(x, self.norm.weight, self.norm.bias, self.gamma, training=True)
+                and ops.usable(shortcut, training=True)):
+            # on the GPU: NCHW -> LayerNorm -> NHWC, and NHWC -> layer scale -> + shortcut -> NCHW, are one kernel
+            # each instead of a layout copy plus an elementwise pass each; where autograd records, through the
+            # functions that carry the backward kernels
+            if ops.records(x, self.norm.weight, self.norm.bias):
+                y = ops.channel_norm_fn(x, self.norm.weight, self.norm.bias, self.norm.eps, True)
+            else:
+                y = ops.channel_norm(x, self.norm.weight, self.norm.bias, self.norm.eps, nhwc=True)
+            y = self.mlp(y)
+            # the MLP may change the dtype; the residual kernels take a tensor of the shortcut's type
             if ops.usable_nhwc(y, shortcut):
-                return ops.block_residual(y.contiguous(), shortcut, self.gamma)
+                y = y.contiguous()
+                if ops.records(y, shortcut, self.gamma):
+                    if self.gamma is not None:
+                        return ops.block_residual_fn(y, shortcut, self.gamma)
+                else:
+                    return ops.block_residual(y, shortcut, self.gamma)
             x = y.permute(0, 3, 1, 2)
         else:
             x = x.permute(0, 2, 3, 1)
