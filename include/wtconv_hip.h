@@ -201,6 +201,16 @@ int wtconv_block_residual_backward(const void* dout, const void* y, const void* 
                                    int B, int C, int HW, int dtype, int param_dtype, void* workspace,
                                    size_t workspace_bytes, void* stream);
 
+/* ---- single-level Haar (db1) transforms as operators of their own: wavelet_2d_transform /
+ * inverse_2d_wavelet_transform and their 1-D twins with the db1 bank (wtconv/util/wavelet.py:46-75; the fast
+ * twin's haar2d / ihaar2d utilities, fast_wtconv/cuda_haar/__init__.py:52-55).  Even extents only (the reference
+ * pads before it calls them, wtconv2d.py:49-51).
+ *   wtconv_haar2d, inverse == 0: x (planes, H, W) -> out (planes, 4, H/2, W/2), sub-bands LL, LH, HL, HH;
+ *                  inverse != 0: x (planes, 4, H/2, W/2) -> out (planes, H, W).
+ *   wtconv_haar1d, inverse == 0: x (rows, N) -> out (rows, 2, N/2), lo then hi; inverse != 0 the other way. */
+int wtconv_haar2d(const void* x, void* out, long long planes, int H, int W, int dtype, int inverse, void* stream);
+int wtconv_haar1d(const void* x, void* out, long long rows, int N, int dtype, int inverse, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,10 +11,11 @@ EMU_DIR = os.path.join(ROOT, "tests", "emu")
 BUILD_DIR = os.path.join(EMU_DIR, "_build")
 EXE = os.path.join(BUILD_DIR, "emu_driver")
 SOURCES = [os.path.join(ROOT, "wtconv_amd", "csrc", "api.hip"), os.path.join(ROOT, "wtconv_amd", "csrc", "mfma2d.hip"),
-           os.path.join(ROOT, "wtconv_amd", "csrc", "block.hip"), os.path.join(EMU_DIR, "emu_driver.cpp")]
+           os.path.join(ROOT, "wtconv_amd", "csrc", "block.hip"), os.path.join(ROOT, "wtconv_amd", "csrc", "haar.hip"),
+           os.path.join(EMU_DIR, "emu_driver.cpp")]
 DEPS = SOURCES + [os.path.join(ROOT, "wtconv_amd", "csrc", f) for f in
                   ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h", "kernels2d_mfma_wgrad.h",
-                   "kernels2d_stream.h", "mfma2d.h", "plan.h", "kernels_block.h", "wgrad_finish.h")] + [
+                   "kernels2d_stream.h", "mfma2d.h", "plan.h", "kernels_block.h", "kernels_haar.h", "wgrad_finish.h")] + [
     os.path.join(EMU_DIR, "emu_runtime.h"), os.path.join(ROOT, "include", "wtconv_hip.h")]
 
 

@@ -6,8 +6,9 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libwtconv_hip.so")
-SOURCES = [os.path.join(CSRC, "api.hip"), os.path.join(CSRC, "mfma2d.hip"), os.path.join(CSRC, "block.hip")]
-HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h", "kernels2d_mfma_wgrad.h", "kernels_block.h",
+SOURCES = [os.path.join(CSRC, "api.hip"), os.path.join(CSRC, "mfma2d.hip"), os.path.join(CSRC, "block.hip"),
+           os.path.join(CSRC, "haar.hip")]
+HEADERS = [os.path.join(CSRC, f) for f in ("common.h", "host_util.h", "kernels1d.h", "kernels1d_row.h", "kernels2d.h", "kernels2d_mfma.h", "kernels2d_mfma_wgrad.h", "kernels_block.h", "kernels_haar.h", "wgrad_finish.h",
                                          "kernels2d_stream.h", "mfma2d.h", "plan.h")] + [
     os.path.join(os.path.dirname(PKG_DIR), "include", "wtconv_hip.h")]
 

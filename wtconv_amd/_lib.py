@@ -50,6 +50,10 @@ EXPORTS["wtconv_block_workspace_bytes"] = (_z, [_i, _i, _i, _i])
 EXPORTS["wtconv_channel_norm_backward"] = (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _i, _p, _z, _p])
 EXPORTS["wtconv_block_residual_backward"] = (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _z, _p])
 
+_ll = ctypes.c_longlong
+EXPORTS["wtconv_haar2d"] = (_i, [_p, _p, _ll, _i, _i, _i, _i, _p])
+EXPORTS["wtconv_haar1d"] = (_i, [_p, _p, _ll, _i, _i, _i, _p])
+
 _lib = None
 _lock = threading.Lock()
 
