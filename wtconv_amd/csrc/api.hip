@@ -82,7 +82,6 @@ static int run_plane2d_mode(const void* x, void* out, const float* fw, const flo
 template <typename T>
 static int run_plane2d_static(int K, int tj1, const void* x, void* out, const float* fw, const float* fb,
                               const Plan2D& pl, hipStream_t stream) {
-#ifndef WT_EMULATE
   if (K != 5 || pl.H != pl.W) return 1;
 #define WT_TRY(H_, L_)                                                                                  \
   if (pl.H == H_ && pl.L == L_) {                                                                       \
@@ -94,7 +93,6 @@ static int run_plane2d_static(int K, int tj1, const void* x, void* out, const fl
   }
   WT_TRY(56, 3) WT_TRY(28, 3) WT_TRY(14, 2) WT_TRY(7, 2)
 #undef WT_TRY
-#endif
   return 1;
 }
 
@@ -145,7 +143,6 @@ static int run_wgrad2d(const void* x, const void* g, float* partial, const Plan2
 template <typename T>
 static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float* partial, const Plan2D& pl, int B,
                               int bchunk, int nchunk, const FinishArgs& fin, hipStream_t stream) {
-#ifndef WT_EMULATE
   if (K != 5 || pl.H != pl.W) return 1;
 #define WT_TRY(H_, L_)                                                                                   \
   if (pl.H == H_ && L == L_) {                                                                           \
@@ -158,7 +155,6 @@ static int run_wgrad2d_static(int K, int L, const void* x, const void* g, float*
   }
   WT_TRY(56, 3) WT_TRY(28, 3) WT_TRY(14, 2) WT_TRY(7, 2)
 #undef WT_TRY
-#endif
   return 1;
 }
 

@@ -31,6 +31,7 @@ constexpr int kDivShift = 20;        // magic reciprocals: exact for dividends <
 struct MPlan {
   int B, C, H, W, L;
   int pb, upc, nunits;               // planes (one channel, consecutive batch items) per unit; units per channel; total
+  int bq, br;                        // B = upc * bq + br: the first br units of a channel take bq + 1 batch items, the rest bq
   int nfilt;                         // 1 + 4 L
   int h[kMaxLevels + 1], w[kMaxLevels + 1];        // extent of level l (0 = pixels)
   int nbr[kMaxLevels + 1], nbc[kMaxLevels + 1];    // 4x4 blocks per plane: rows, columns
@@ -449,7 +450,7 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
     if constexpr (Geo::kStatic) {
       constexpr MPlan g = Geo::template plan<NS>();
       MPlan p = g;
-      p.B = plarg.B; p.C = plarg.C; p.upc = plarg.upc; p.nunits = plarg.nunits;
+      p.B = plarg.B; p.C = plarg.C; p.upc = plarg.upc; p.nunits = plarg.nunits; p.bq = plarg.bq; p.br = plarg.br;
       return p;
     } else {
       return plarg;
@@ -526,12 +527,13 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   const size_t total_elems = static_cast<size_t>(B) * C * HW;
   auto fetch = [&](int u) {
     const int c = u / upc;
-    const int b0 = (u - c * upc) * pb;
+    const int ubf = u - c * upc;
+    const int b0 = ubf * pl.bq + (ubf < pl.br ? ubf : pl.br);      // the batch is spread evenly over the channel's units (see below)
     const size_t base_off = (static_cast<size_t>(b0) * C + c) * HW;
     const T* base = x + base_off;
 #pragma unroll
     for (int i = 0; i < NBL; ++i) {
-      const bool plane_ok = (c_mask[i] & 0x100u) && b0 + c_p[i] < B;
+      const bool plane_ok = (c_mask[i] & 0x100u) && c_p[i] < pl.bq + (ubf < pl.br ? 1 : 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         pix_zero(pf[i][r]);
@@ -567,8 +569,11 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
 #pragma unroll 1
   for (int u = u_begin; u < u_end; ++u) {
     const int c = u / upc;
-    const int b0 = (u - c * upc) * pb;
-    const int np = B - b0 < pb ? B - b0 : pb;      // planes of this unit that exist
+    // The batch is spread evenly over the units of a channel: at most pb items each, all units within one plane of
+    // each other (a short last unit would leave the workgroups that get it with less work than the rest).
+    const int ub = u - c * upc;
+    const int b0 = ub * pl.bq + (ub < pl.br ? ub : pl.br);
+    const int np = pl.bq + (ub < pl.br ? 1 : 0);   // planes of this unit that exist
     if (c != cur_c) {     // (the previous unit ended with a barrier: nobody still reads the old table)
       // fold this channel's parameters into the fragment table: filters from `tfirst` on into their
       // LDS table, the ones before it (held in registers) through the idle Z_1 buffer

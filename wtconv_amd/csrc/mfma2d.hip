@@ -20,6 +20,8 @@ bool make_mplan(int B, int C, int H, int W, int L, int NS, int pb, MPlan* out) {
   if (!make_mplan_geometry(H, W, L, NS, pb, out)) return false;
   out->B = B; out->C = C;
   out->upc = ceil_div(B, pb);
+  out->bq = B / out->upc;
+  out->br = B % out->upc;
   if (static_cast<long long>(C) * out->upc > 0x7fffffffLL) return false;
   out->nunits = C * out->upc;
   if (static_cast<long long>(pb) * C * H * W > 0x7fffffffLL) return false;
