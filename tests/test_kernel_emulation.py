@@ -106,6 +106,21 @@ def test_emulated_2d_level_by_level(B, C, H, W, K, L, bias, limit):
     _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5)
 
 
+@pytest.mark.parametrize("B,C,H,W,K,L,bias,limit,dtype", [
+    (2, 2, 21, 37, 5, 3, True, 1024, 0),     # both passes level by level: one pyramid of grad_out serves both
+    (1, 1, 24, 48, 3, 2, False, 1024, 2),    # the same on fp16 tensors
+    (1, 1, 18, 24, 7, 1, True, 1024, 0),     # a single level: nothing to share, the two passes run as they are
+    (1, 1, 36, 36, 3, 2, False, 12000, 0),   # plane-resident input gradient, level-by-level weight gradients: not shared
+    (2, 3, 14, 14, 5, 2, True, None, 0),     # plane-resident both: the plain sequence of the two passes
+])
+def test_emulated_2d_fused_backward(B, C, H, W, K, L, bias, limit, dtype):
+    """wtconv2d_backward as one call, against the oracle (and so against the two separate passes)."""
+    x, g, bw, bb, bs, ws, ss = _case2d(B, C, H, W, K, L, bias, dtype=dtype)
+    got = emu_util.run(2, x, g, bw, bb, bs, ws, ss, K, dtype=dtype, lds_limit=limit, fused_bwd=True)
+    act = (1e-3, 1e-3) if dtype == 2 else None
+    _compare(got, _oracle(2, x, g, bw, bb, bs, ws, ss), rtol=2e-5, atol_scale=2e-5, act_tol=act)
+
+
 # A single tiny plane: the pyramids take less LDS than the final reduction of the
 # weight-gradient kernel ([8 waves][sets * K * K + 1] floats), which the plan must cover.
 @pytest.mark.parametrize("B,C,H,W,K,L", [

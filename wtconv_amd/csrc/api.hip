@@ -264,12 +264,13 @@ static int stream_analysis_chain(const T* src, float* pyr, const Stream2D& sp, h
   return 0;
 }
 
+// `have_pyramid`: the pyramid of x is in `pyr` already (the whole backward pass shares the one of grad_out).
 template <typename T, int K>
 static int run_stream2d(const void* x_, void* out_, const float* fw, const float* fb, float* pyr, const Stream2D& sp,
-                        hipStream_t stream) {
+                        hipStream_t stream, bool have_pyramid = false) {
   const T* x = static_cast<const T*>(x_);
   T* out = static_cast<T*>(out_);
-  if (sp.L > 1) {      // a single level is synthesised from the pixels alone
+  if (sp.L > 1 && !have_pyramid) {      // a single level is synthesised from the pixels alone
     if (int e = stream_analysis_chain<T>(x, pyr, sp, stream, true)) return e;
   }
   const unsigned gy = sp.nplanes < 65535 ? sp.nplanes : 65535;
@@ -298,23 +299,25 @@ static int run_stream2d(const void* x_, void* out_, const float* fw, const float
 
 template <typename T>
 static int run_stream2d_k(int K, const void* x, void* out, const float* fw, const float* fb, float* pyr,
-                          const Stream2D& sp, hipStream_t stream) {
+                          const Stream2D& sp, hipStream_t stream, bool have_pyramid = false) {
   switch (K) {
-    case 1: return run_stream2d<T, 1>(x, out, fw, fb, pyr, sp, stream);
-    case 3: return run_stream2d<T, 3>(x, out, fw, fb, pyr, sp, stream);
-    case 5: return run_stream2d<T, 5>(x, out, fw, fb, pyr, sp, stream);
-    case 7: return run_stream2d<T, 7>(x, out, fw, fb, pyr, sp, stream);
+    case 1: return run_stream2d<T, 1>(x, out, fw, fb, pyr, sp, stream, have_pyramid);
+    case 3: return run_stream2d<T, 3>(x, out, fw, fb, pyr, sp, stream, have_pyramid);
+    case 5: return run_stream2d<T, 5>(x, out, fw, fb, pyr, sp, stream, have_pyramid);
+    case 7: return run_stream2d<T, 7>(x, out, fw, fb, pyr, sp, stream, have_pyramid);
   }
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
 
+// `have_g_pyramid`: the pyramid of grad_out is in `pyr_g` already (left there by the input-gradient pass of the same call).
 template <typename T, int K>
 static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, float* pyr_x, float* pyr_g,
-                              const Stream2D& sp, int B, int nchunk, hipStream_t stream) {
+                              const Stream2D& sp, int B, int nchunk, hipStream_t stream, bool have_g_pyramid = false) {
   const T* x = static_cast<const T*>(x_);
   const T* g = static_cast<const T*>(g_);
   if (int e = stream_analysis_chain<T>(x, pyr_x, sp, stream, false)) return e;
-  if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream, false)) return e;
+  if (!have_g_pyramid)
+    if (int e = stream_analysis_chain<T>(g, pyr_g, sp, stream, false)) return e;
   const int rec = (1 + 4 * sp.L) * K * K + 1;
   const bool pyr_ok = aligned16(pyr_x) && aligned16(pyr_g);
   // chunks of a launch: at least four (batch item, tile) units per workgroup where the level has them
@@ -341,19 +344,21 @@ static int run_stream2d_wgrad(const void* x_, const void* g_, float* partial, fl
 
 template <typename T>
 static int run_stream2d_wgrad_k(int K, const void* x, const void* g, float* partial, float* pyr_x, float* pyr_g,
-                                const Stream2D& sp, int B, int nchunk, hipStream_t stream) {
+                                const Stream2D& sp, int B, int nchunk, hipStream_t stream, bool have_g_pyramid = false) {
   switch (K) {
-    case 1: return run_stream2d_wgrad<T, 1>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
-    case 3: return run_stream2d_wgrad<T, 3>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
-    case 5: return run_stream2d_wgrad<T, 5>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
-    case 7: return run_stream2d_wgrad<T, 7>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream);
+    case 1: return run_stream2d_wgrad<T, 1>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream, have_g_pyramid);
+    case 3: return run_stream2d_wgrad<T, 3>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream, have_g_pyramid);
+    case 5: return run_stream2d_wgrad<T, 5>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream, have_g_pyramid);
+    case 7: return run_stream2d_wgrad<T, 7>(x, g, partial, pyr_x, pyr_g, sp, B, nchunk, stream, have_g_pyramid);
   }
   return fail(WTCONV_E_UNSUPPORTED, "kernel_size %d is not built", K);
 }
 
+// `shared_pyr` (level-by-level path only): where to build the whole pyramid of x -- detail bands of level 1 included --
+// for a later pass of the same call to reuse; the folded parameters then go to `shared_fw` instead of the workspace start.
 static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
                         int H, int W, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes,
-                        void* stream_, int flip) {
+                        void* stream_, int flip, float* shared_pyr = nullptr, float* shared_fw = nullptr) {
   if (int e = check_common(fn, params, B, C, K, L, dtype, pdtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
   if (static_cast<long long>(H) * W > kMaxPlaneElems)   // 32-bit offsets inside a plane and its four stacked sub-bands
@@ -372,11 +377,14 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
     return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, stream, flip);
   if (!plane_fits_lds(B, C, H, W, K, L)) {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
-    float* fw = static_cast<float*>(ws);
+    float* fw = shared_pyr != nullptr ? shared_fw : static_cast<float*>(ws);
     float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
-    float* pyr = fw + round_up64(fold_floats(C, 4, L, K * K));
+    float* pyr = shared_pyr != nullptr ? shared_pyr : fw + round_up64(fold_floats(C, 4, L, K * K));
     if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
-    return WT_BY_DTYPE(dtype, run_stream2d_k<T_>(K, x, out, fw, fb, pyr, sp, stream));
+    if (shared_pyr != nullptr) {
+      if (int e = WT_BY_DTYPE(dtype, stream_analysis_chain<T_>(static_cast<const T_*>(x), pyr, sp, stream, false))) return e;
+    }
+    return WT_BY_DTYPE(dtype, run_stream2d_k<T_>(K, x, out, fw, fb, pyr, sp, stream, shared_pyr != nullptr));
   }
   Plan2D pl = make_plan2d(B, C, H, W, K, L, false, 256, esz, x, out, nullptr);
   int tj1 = 4, sg_shift = 8;
@@ -772,11 +780,11 @@ int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_par
                       param_dtype, workspace, workspace_bytes, stream, 1);
 }
 
-int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+// have_g_pyramid (level-by-level path only): the pyramid of grad_out is in its place in the workspace already.
+static int backward_params2d(const char* fn, const void* x, const void* grad_out, const wtconv_params* params,
                              const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels,
                              int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
-                             void* stream_) {
-  const char* fn = "wtconv2d_backward_params";
+                             void* stream_, bool have_g_pyramid) {
   const int L = levels;
   if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
@@ -833,7 +841,8 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
     if (nchunk > 65535 || C > 0x7fffffff / 4) return fail(WTCONV_E_UNSUPPORTED, "%s: too many chunks (%d)", fn, nchunk);
     float* pyr_x = partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * L) * K * K + 1));
     float* pyr_g = pyr_x + sp.floats;
-    e = WT_BY_DTYPE(dtype, run_stream2d_wgrad_k<T_>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream));
+    e = WT_BY_DTYPE(dtype, run_stream2d_wgrad_k<T_>(K, x, grad_out, partial, pyr_x, pyr_g, sp, B, nchunk, stream,
+                                                    have_g_pyramid));
   }
   if (e || resident) return e;
   const GradTable gt = to_grad_table(grads, L);
@@ -843,10 +852,41 @@ int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_p
   return check_launch("wgrad_finish_kernel");
 }
 
+int wtconv2d_backward_params(const void* x, const void* grad_out, const wtconv_params* params,
+                             const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels,
+                             int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  return backward_params2d("wtconv2d_backward_params", x, grad_out, params, grads, B, C, H, W, K, levels, dtype,
+                           param_dtype, workspace, workspace_bytes, stream, false);
+}
+
 int wtconv2d_backward(const void* x, const void* grad_out, void* grad_x, const wtconv_params* params,
                       const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels, int dtype,
                       int param_dtype, void* workspace, size_t workspace_bytes, void* stream) {
-  // the two passes run one after the other on the stream and may share the workspace
+  // Planes beyond LDS (both passes level by level): the pyramid of grad_out is built once, in the place the
+  // parameter-gradient pass keeps it, and serves both passes; the folded parameters of the input-gradient pass sit
+  // where the pyramid of x goes afterwards.
+  const bool sizes_ok = B > 0 && C > 0 && H > 0 && W > 0 && K >= 1 && K % 2 == 1 && K <= wtconv_max_kernel_size() &&
+                        levels >= 2 && levels <= kMaxLevels && static_cast<long long>(H) * W <= kMaxPlaneElems;
+  if (sizes_ok && !mfma2d_query(B, C, H, W, K, levels, dtype).ok && !plane_fits_lds(B, C, H, W, K, levels) &&
+      !mfma2d_wgrad_query(B, C, H, W, K, levels, dtype).ok && !wgrad_fits_lds(B, C, H, W, K, levels)) {
+    const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, levels, WTCONV_PASS_BACKWARD);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(WTCONV_E_WORKSPACE, "wtconv2d_backward: workspace of %zu B needed, %zu given", need, workspace_bytes);
+    const Stream2D sp = make_stream2d(B, C, H, W, levels);
+    const int nchunk = stream_chunks(B, C, H, W);
+    float* partial = static_cast<float*>(workspace);
+    float* pyr_x = partial + round_up64(static_cast<size_t>(nchunk) * C * ((1 + 4 * levels) * K * K + 1));
+    float* pyr_g = pyr_x + sp.floats;
+    if (fold_floats(C, 4, levels, K * K) <= sp.floats) {
+      if (int e = plane2d_pass("wtconv2d_backward", grad_out, grad_x, params, B, C, H, W, K, levels, dtype, param_dtype,
+                               workspace, workspace_bytes, stream, 1, pyr_g, pyr_x))
+        return e;
+      return backward_params2d("wtconv2d_backward", x, grad_out, params, grads, B, C, H, W, K, levels, dtype,
+                               param_dtype, workspace, workspace_bytes, stream, true);
+    }
+  }
+  // otherwise the two passes run one after the other on the stream and share the workspace
   if (int e = wtconv2d_backward_input(grad_out, grad_x, params, B, C, H, W, K, levels, dtype, param_dtype, workspace,
                                       workspace_bytes, stream))
     return e;
