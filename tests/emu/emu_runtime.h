@@ -56,20 +56,23 @@ inline void __syncthreads() { emu::tls_block->bar->arrive_and_wait(); }
 inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
 inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
 
-// Every thread of the block must call this the same number of times (true for the
-// kernels here: reductions sit outside divergent code).
+namespace emu {
+// Barrier over the 64 threads of the calling thread's wavefront.
+inline void wave_barrier() { tls_block->wave_bar[threadIdx.x / 64]->arrive_and_wait(); }
+}  // namespace emu
+
+// Every thread of the wavefront must call this the same number of times (true for the kernels here: reductions sit
+// outside divergent code).  Lanes exchange within their wavefront only (mask < 64), so its barrier is enough.
 inline float __shfl_xor(float v, int mask, int /*width*/) {
   emu::BlockState* b = emu::tls_block;
   b->xchg[threadIdx.x] = v;
-  b->bar->arrive_and_wait();
+  emu::wave_barrier();
   const float r = b->xchg[threadIdx.x ^ static_cast<unsigned>(mask)];
-  b->bar->arrive_and_wait();
+  emu::wave_barrier();
   return r;
 }
 
 namespace emu {
-// Barrier over the 64 threads of the calling thread's wavefront.
-inline void wave_barrier() { tls_block->wave_bar[threadIdx.x / 64]->arrive_and_wait(); }
 
 // D = A (16x32) * B (32x16) + C on bfloat16 operands with float accumulation, operands and
 // result distributed over the 64 lanes of a wavefront as v_mfma_f32_16x16x32_bf16 holds them:

@@ -25,11 +25,20 @@ def build(force=False):
         newest = max(os.path.getmtime(p) for p in DEPS)
         if os.path.getmtime(EXE) >= newest:
             return EXE
-    # -O0 -g1: the run time is dominated by thread creation, the build time by optimisation
-    cmd = ["g++", "-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined",
-           "-fno-sanitize-recover=undefined", "-static-libasan", "-DWT_EMULATE", "-I" + EMU_DIR, "-x", "c++",
-           *SOURCES, "-pthread", "-o", EXE]
-    subprocess.run(cmd, check=True, cwd=ROOT)
+    # -O0 -g1: the run time is dominated by thread creation, the build time by optimisation.  One object per source,
+    # compiled side by side.
+    flags = ["-std=c++20", "-O0", "-g1", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+             "-DWT_EMULATE", "-I" + EMU_DIR, "-pthread"]
+    objs, procs = [], []
+    for src in SOURCES:
+        obj = os.path.join(BUILD_DIR, os.path.basename(src) + ".o")
+        objs.append(obj)
+        procs.append(subprocess.Popen(["g++", *flags, "-x", "c++", "-c", src, "-o", obj], cwd=ROOT))
+    failed = [src for src, pr in zip(SOURCES, procs) if pr.wait() != 0]
+    if failed:
+        raise RuntimeError("emulation build failed for " + ", ".join(failed))
+    subprocess.run(["g++", "-fsanitize=address,undefined", "-static-libasan", "-pthread", *objs, "-o", EXE], check=True,
+                   cwd=ROOT)
     return EXE
 
 

@@ -107,7 +107,7 @@ def test_emulated_2d_level_by_level(B, C, H, W, K, L, bias, limit):
 
 
 @pytest.mark.parametrize("B,C,H,W,K,L,bias,limit,dtype", [
-    (2, 2, 21, 37, 5, 3, True, 1024, 0),     # both passes level by level: one pyramid of grad_out serves both
+    (1, 2, 21, 37, 5, 3, True, 1024, 0),     # both passes level by level: one pyramid of grad_out serves both
     (1, 1, 24, 48, 3, 2, False, 1024, 2),    # the same on fp16 tensors
     (1, 1, 18, 24, 7, 1, True, 1024, 0),     # a single level: nothing to share, the two passes run as they are
     (1, 1, 36, 36, 3, 2, False, 12000, 0),   # plane-resident input gradient, level-by-level weight gradients: not shared
@@ -265,8 +265,7 @@ def _case1d(B, C, N, K, L, bias, seed=0):
     (1, 1, 700, 7, 3, False),      # row-resident, K = 7: level 3 holds 2 < R entries per lane
     (1, 1, 600, 3, 5, True),       # row-resident, five levels
     (1, 1, 800, 5, 5, True),       # row-resident, one level-5 entry per lane: edges from two lanes away
-    (1, 1, 17000, 5, 4, True),     # longer than 512 lanes: tiled kernels, 17 tiles
-])
+])                                 # (rows beyond 512 lanes, on the tiled kernels: test_emulated_1d_fused_backward)
 def test_emulated_1d_fp32(B, C, N, K, L, bias):
     x, g, bw, bb, bs, ws, ss = _case1d(B, C, N, K, L, bias)
     got = emu_util.run(1, x, g, bw, bb, bs, ws, ss, K)
@@ -296,7 +295,7 @@ def test_emulated_1d_row_resident_bf16():
     (1, 1, 700, 7, 3, True, 0, 0),       # K = 7
     (1, 2, 800, 3, 5, True, 0, 0),       # five levels
     (2, 1, 1000, 5, 4, True, 1, 1),      # bf16 rows and parameters
-    (1, 1, 17000, 5, 4, True, 0, 0),     # longer than the fused kernel takes: falls back to the two half passes
+    (1, 1, 17000, 5, 4, True, 0, 0),     # longer than 512 lanes: every pass on the tiled kernels (17 tiles)
 ])
 def test_emulated_1d_fused_backward(B, C, N, K, L, bias, dtype, pdtype):
     """wtconv1d_backward as one call: grad_x and every parameter gradient from the fused row kernel (the last

@@ -52,12 +52,13 @@ constexpr int kWgradResident = 512;
 static size_t fold_floats(int C, int S, int L, int KK) { return static_cast<size_t>(C) * (1 + S * L) * KK + C; }
 
 static int launch_fold(const wtconv_params* params, int pdtype, float* fw, float* fb, int C, int S, int L,
-                       int KK, int flip, int use_bias, hipStream_t stream) {
+                       int KK, int flip, int use_bias, hipStream_t stream, unsigned* zero_words = nullptr,
+                       int nzero = 0) {
   const int total = C * (1 + S * L) * KK;
   int blocks = (total + 255) / 256;
   if (blocks > 1024) blocks = 1024;
   WT_LAUNCH(fold_params_kernel, dim3(blocks), dim3(256), 0, stream, to_table(params, L), pdtype, fw, fb, C, S, L,
-            KK, flip, use_bias);
+            KK, flip, use_bias, zero_words, zero_words != nullptr ? nzero : 0);
   return check_launch("fold_params_kernel");
 }
 
@@ -356,9 +357,12 @@ static int run_stream2d_wgrad_k(int K, const void* x, const void* g, float* part
 
 // `shared_pyr` (level-by-level path only): where to build the whole pyramid of x -- detail bands of level 1 included --
 // for a later pass of the same call to reuse; the folded parameters then go to `shared_fw` instead of the workspace start.
+// `tickets` (plane-resident paths only): C words this pass clears on its way, for the parameter-gradient pass that
+// follows it on the stream; they must lie outside the folded parameters at the workspace start.
 static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C,
                         int H, int W, int K, int L, int dtype, int pdtype, void* ws, size_t ws_bytes,
-                        void* stream_, int flip, float* shared_pyr = nullptr, float* shared_fw = nullptr) {
+                        void* stream_, int flip, float* shared_pyr = nullptr, float* shared_fw = nullptr,
+                        unsigned* tickets = nullptr) {
   if (int e = check_common(fn, params, B, C, K, L, dtype, pdtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
   if (static_cast<long long>(H) * W > kMaxPlaneElems)   // 32-bit offsets inside a plane and its four stacked sub-bands
@@ -374,7 +378,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
   if (static_cast<long long>(B) * C > 0x7fffffffLL / 4)
     return fail(WTCONV_E_UNSUPPORTED, "%s: batch*channels = %lld is too large", fn, static_cast<long long>(B) * C);
   if (mfma2d_query(B, C, H, W, K, L, dtype).ok)
-    return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, stream, flip);
+    return mfma2d_pass(fn, x, out, params, B, C, H, W, K, L, dtype, pdtype, stream, flip, tickets, C);
   if (!plane_fits_lds(B, C, H, W, K, L)) {
     const Stream2D sp = make_stream2d(B, C, H, W, L);
     float* fw = shared_pyr != nullptr ? shared_fw : static_cast<float*>(ws);
@@ -398,7 +402,7 @@ static int plane2d_pass(const char* fn, const void* x, void* out, const wtconv_p
                 "plane-resident kernels", fn, H, W, L, static_cast<size_t>(pl.lds_floats) * 4, kLdsLimitBytes);
   float* fw = static_cast<float*>(ws);
   float* fb = fw + static_cast<size_t>(C) * (1 + 4 * L) * K * K;
-  if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream)) return e;
+  if (int e = launch_fold(params, pdtype, fw, fb, C, 4, L, K * K, flip, flip ? 0 : 1, stream, tickets, C)) return e;
   if (dtype != WTCONV_BF16) {     // (bf16 tensors of these shapes are on the matrix-core kernels)
     const int e = dtype == WTCONV_F32 ? run_plane2d_static<float>(K, tj1, x, out, fw, fb, pl, stream)
                                       : run_plane2d_static<f16_t>(K, tj1, x, out, fw, fb, pl, stream);
@@ -780,11 +784,18 @@ int wtconv2d_backward_input(const void* grad_out, void* grad_x, const wtconv_par
                       param_dtype, workspace, workspace_bytes, stream, 1);
 }
 
+// Where the parameter-gradient pass of a plane-resident shape keeps its channel tickets in the workspace.
+static unsigned* wgrad2d_tickets(void* workspace, int B, int C, int H, int W, int K, int L) {
+  const size_t need = wtconv2d_workspace_bytes(B, C, H, W, K, L, WTCONV_PASS_BACKWARD_PARAMS);
+  return reinterpret_cast<unsigned*>(static_cast<char*>(workspace) + need) - C;
+}
+
 // have_g_pyramid (level-by-level path only): the pyramid of grad_out is in its place in the workspace already.
+// tickets_zeroed (plane-resident paths only): an earlier kernel on the stream has cleared the channel tickets.
 static int backward_params2d(const char* fn, const void* x, const void* grad_out, const wtconv_params* params,
                              const wtconv_param_grads* grads, int B, int C, int H, int W, int K, int levels,
                              int dtype, int param_dtype, void* workspace, size_t workspace_bytes,
-                             void* stream_, bool have_g_pyramid) {
+                             void* stream_, bool have_g_pyramid, bool tickets_zeroed = false) {
   const int L = levels;
   if (int e = check_common(fn, params, B, C, K, L, dtype, param_dtype)) return e;
   if (H <= 0 || W <= 0) return fail(WTCONV_E_ARG, "%s: spatial size must be positive (got %dx%d)", fn, H, W);
@@ -815,12 +826,14 @@ static int backward_params2d(const char* fn, const void* x, const void* grad_out
   // word per channel at the end of the workspace, cleared by a small launch of its own.
   FinishArgs fin = {};
   if (resident) {
-    fin.tickets = reinterpret_cast<unsigned*>(static_cast<char*>(workspace) + need) - C;
+    fin.tickets = wgrad2d_tickets(workspace, B, C, H, W, K, L);
     fin.prm = to_table(params, L);
     fin.pdtype = param_dtype;
     fin.gt = to_grad_table(grads, L);
-    WT_LAUNCH(zero_tickets_kernel, dim3((C + 255) / 256), dim3(256), 0, stream, fin.tickets, C);
-    if (int ze = check_launch("zero_tickets_kernel")) return ze;
+    if (!tickets_zeroed) {
+      WT_LAUNCH(zero_tickets_kernel, dim3((C + 255) / 256), dim3(256), 0, stream, fin.tickets, C);
+      if (int ze = check_launch("zero_tickets_kernel")) return ze;
+    }
   }
   if (mq.ok) {
     nchunk = mq.nchunk;
@@ -886,7 +899,23 @@ int wtconv2d_backward(const void* x, const void* grad_out, void* grad_x, const w
                                param_dtype, workspace, workspace_bytes, stream, true);
     }
   }
-  // otherwise the two passes run one after the other on the stream and share the workspace
+  // Otherwise the two passes run one after the other on the stream and share the workspace.  Plane-resident shapes:
+  // the input-gradient pass clears the channel tickets of the parameter-gradient pass on its way (one launch fewer),
+  // where they lie beyond the folded parameters that it keeps at the start of the workspace.
+  if (sizes_ok && workspace != nullptr &&
+      workspace_bytes >= wtconv2d_workspace_bytes(B, C, H, W, K, levels, WTCONV_PASS_BACKWARD) &&
+      (mfma2d_query(B, C, H, W, K, levels, dtype).ok || plane_fits_lds(B, C, H, W, K, levels)) &&
+      (mfma2d_wgrad_query(B, C, H, W, K, levels, dtype).ok || wgrad_fits_lds(B, C, H, W, K, levels))) {
+    unsigned* tickets = wgrad2d_tickets(workspace, B, C, H, W, K, levels);
+    const char* fold_end = static_cast<const char*>(workspace) + fold_floats(C, 4, levels, K * K) * sizeof(float);
+    if (reinterpret_cast<const char*>(tickets) >= fold_end) {
+      if (int e = plane2d_pass("wtconv2d_backward", grad_out, grad_x, params, B, C, H, W, K, levels, dtype, param_dtype,
+                               workspace, workspace_bytes, stream, 1, nullptr, nullptr, tickets))
+        return e;
+      return backward_params2d("wtconv2d_backward", x, grad_out, params, grads, B, C, H, W, K, levels, dtype,
+                               param_dtype, workspace, workspace_bytes, stream, false, true);
+    }
+  }
   if (int e = wtconv2d_backward_input(grad_out, grad_x, params, B, C, H, W, K, levels, dtype, param_dtype, workspace,
                                       workspace_bytes, stream))
     return e;

@@ -54,12 +54,14 @@ struct Plan2D {
 
 // ------------------------------------------------------------------ parameter folding
 // fw[c][f][t]: f = 0 base conv, f = 1 + S*l + s level l sub-band s; value gamma * w, taps
-// reversed when flip != 0.  fb[c] = gamma_b * bias (0 without bias).
+// reversed when flip != 0.  fb[c] = gamma_b * bias (0 without bias).  Also clears the `nzero` words at `zero_words`
+// (the channel tickets of a parameter-gradient pass that follows on the stream).
 __global__ void fold_params_kernel(ParamTable p, int pdtype, float* __restrict__ fw,
                                    float* __restrict__ fb, int C, int S, int L, int KK,
-                                   int flip, int use_bias) {
+                                   int flip, int use_bias, unsigned* __restrict__ zero_words, int nzero) {
   const int NF = 1 + S * L;
   const int total = C * NF * KK;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nzero; i += gridDim.x * blockDim.x) zero_words[i] = 0u;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     const int t = idx % KK;
     const int f = (idx / KK) % NF;

@@ -444,7 +444,7 @@ __device__ __forceinline__ TileLane tile_lane(const char* lds, int T, int n, int
 template <typename T, int NS, int NBL, bool VEC, bool RES, typename Geo>
 __global__ void __launch_bounds__(kMfmaBlock, NS == 1 ? 4 : 2)      // waves per SIMD the register budget must allow
 wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable prm, int pdtype, int K, int flip,
-                 int use_bias, const MPlan plarg) {
+                 int use_bias, const MPlan plarg, unsigned* __restrict__ zero_words, int nzero) {
   // the plan: shape-dependent fields from the compile-time constant where there is one
   const MPlan pl = [&]() {
     if constexpr (Geo::kStatic) {
@@ -462,6 +462,9 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   const int n = lane & 15, q = lane >> 4;
   const int L = pl.L, H = pl.H, W = pl.W;
   const int HW = H * W;
+  // the channel tickets of a parameter-gradient pass that follows on the stream
+  if (blockIdx.x == 0)
+    for (int i = tid; i < nzero; i += kMfmaBlock) zero_words[i] = 0u;
 
   // Toeplitz fragment entries of this lane: output (row ar, column ac) of a block, patch row q (+4)
   const int ar = n >> 2, ac = n & 3;

@@ -17,9 +17,10 @@ struct Mfma2dQuery {
 Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype);
 
 // One pass (flip = 0: forward, 1: input gradient).  Returns 0 or a WTCONV_E_* code with the
-// message left in the thread's error buffer.
+// message left in the thread's error buffer.  The kernel also clears the `nzero` words at `zero_words` (may be null).
 int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
-                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip);
+                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip, unsigned* zero_words = nullptr,
+                int nzero = 0);
 
 // Parameter gradients of bf16 tensors: whether the shape runs on the MFMA kernel, and the size of the
 // per-chunk partial sums it leaves in the workspace (`nchunk` records per channel).

@@ -117,6 +117,8 @@ bool choose_mplan_uncached(int B, int C, int H, int W, int L, int NS, MPlan* out
 struct MfmaArgs {
   ParamTable prm;
   int pdtype, K, flip, use_bias;
+  unsigned* zero_words;
+  int nzero;
 };
 
 template <typename T, int NS, int NBL, bool VEC, typename Geo>
@@ -127,7 +129,7 @@ int launch_mfma(const void* x, void* out, const MfmaArgs& a, const MPlan& pl, hi
   int nwg = compute_units() * resident_per_cu(kern, kMfmaBlock, lds);
   if (nwg > pl.nunits) nwg = pl.nunits;
   WT_LAUNCH(kern, dim3(nwg), dim3(kMfmaBlock), lds, stream, static_cast<const T*>(x), static_cast<T*>(out), a.prm,
-            a.pdtype, a.K, a.flip, a.use_bias, pl);
+            a.pdtype, a.K, a.flip, a.use_bias, pl, a.zero_words, a.nzero);
   return check_launch("wt2d_mfma_kernel");
 }
 
@@ -187,13 +189,13 @@ Mfma2dQuery mfma2d_query(int B, int C, int H, int W, int K, int L, int dtype) {
 }
 
 int mfma2d_pass(const char* fn, const void* x, void* out, const wtconv_params* params, int B, int C, int H, int W,
-                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip) {
+                int K, int L, int dtype, int pdtype, hipStream_t stream, int flip, unsigned* zero_words, int nzero) {
   const int NS = dtype == WTCONV_F32 ? 3 : 1;
   MPlan pl;
   int nbl;
   if (!choose_mplan(B, C, H, W, L, NS, &pl, &nbl))
     return fail(WTCONV_E_UNSUPPORTED, "%s: shape not covered by the matrix-core kernels", fn);
-  const MfmaArgs a = {to_table(params, L), pdtype, K, flip, flip ? 0 : 1};
+  const MfmaArgs a = {to_table(params, L), pdtype, K, flip, flip ? 0 : 1, zero_words, zero_words != nullptr ? nzero : 0};
   const size_t esz = dtype == WTCONV_F32 ? 4 : 2;
   const uintptr_t mask = 4 * esz - 1;
   const bool vec = (W % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & mask) == 0 &&
