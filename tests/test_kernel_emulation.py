@@ -317,7 +317,9 @@ def test_emulated_1d_fused_backward(B, C, N, K, L, bias, dtype, pdtype):
     (1, 10, 9, 13, 0, 0, 0),      # NCHW output (LayerNorm2d), two tiles
     (2, 4, 1, 1, 0, 0, 1),        # a single pixel
     (1, 96, 6, 6, 1, 1, 1),       # bf16 tensors and parameters, 4-element vector rows
-    (1, 24, 8, 10, 1, 0, 0),      # bf16 tensors (tile of floats forward), fp32 parameters
+    (1, 24, 8, 10, 1, 0, 0),      # bf16 tensors, fp32 parameters, NCHW output from registers
+    (2, 10, 4, 6, 0, 0, 1),       # fp32 vector rows: five channel pairs over 32 pair slots, two-dword pair words
+    (1, 200, 4, 4, 1, 0, 1),      # 100 channel pairs: four pixel groups per tile, four pairs per thread, idle slots
 ])
 def test_emulated_channel_norm(B, C, H, W, dtype, pdtype, nhwc):
     """wtconv_channel_norm and its backward on the host under the sanitizers, against torch in float64."""
@@ -342,7 +344,8 @@ def test_emulated_channel_norm(B, C, H, W, dtype, pdtype, nhwc):
     np.testing.assert_allclose(db, tb.grad.numpy(), rtol=tol, atol=tol * max(1.0, float(np.abs(tb.grad.numpy()).max())))
 
 
-@pytest.mark.parametrize("B,C,H,W,dtype", [(2, 6, 5, 3, 0), (1, 10, 9, 13, 0), (2, 4, 1, 1, 0), (1, 96, 6, 6, 1)])
+@pytest.mark.parametrize("B,C,H,W,dtype", [(2, 6, 5, 3, 0), (1, 10, 9, 13, 0), (2, 4, 1, 1, 0), (1, 96, 6, 6, 1),
+                                           (2, 10, 4, 6, 0), (1, 200, 4, 4, 1)])     # the last three: vector rows
 def test_emulated_block_residual(B, C, H, W, dtype):
     """wtconv_block_residual and its backward on the host under the sanitizers, against torch in float64."""
     rng = np.random.default_rng(B * 7 + C)

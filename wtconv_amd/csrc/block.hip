@@ -68,6 +68,65 @@ const TileVal& block_tile_cached(int C, int HW, int esz, int ntile = 1) {
   return it->second;
 }
 
+// Plan of the register-resident channel norm (channel_norm_reg_kernel): G pixel groups of four per tile so that a thread
+// holds at most `np_max` channel pairs; the padding of the pixel-major LDS tile that spreads a wave's writes best over
+// the banks.  false: too many channels for the registers of a workgroup (the LDS-tile kernel takes the call).
+constexpr int kNormPairs = 6;
+
+bool make_norm_tile(int C, int HW, size_t esz, NormTile* out, size_t* lds_bytes) {
+  const int C2 = C / 2, pw = static_cast<int>(esz) / 2;           // dwords per channel pair
+  int gshift = 5;
+  while (gshift > 0 && (static_cast<long long>(C2) << gshift) > 256LL * kNormPairs) --gshift;
+  if (gshift < 1) return false;
+  while (gshift > 1 && (2 << gshift) >= HW) --gshift;             // tiny images: no tile of which half is outside
+  const int cd = C2 * pw;
+  NormTile t = {};
+  auto bytes = [&](int gs, int pd) { return (static_cast<size_t>(4 << gs) * pd + 8 * (4 << gs) + 2 * static_cast<size_t>(C)) * sizeof(float); };
+  while (gshift > 1 && bytes(gshift, cd + 32) > 64 * 1024) --gshift;
+  if (bytes(gshift, cd + 32) > static_cast<size_t>(kLdsLimitBytes)) return false;
+  const int G = 1 << gshift;
+  int best_pad = 0, best = 1 << 30;
+  for (int pad = 0; pad < 32; ++pad) {
+    int cnt[64] = {0};
+    int worst = 0;
+    for (int l = 0; l < 64; ++l) {
+      const int g = l & (G - 1), e = l >> gshift;
+      for (int d = 0; d < pw; ++d) {
+        const int bank = (4 * g * (cd + pad) + e * pw + d) & 63;
+        if (++cnt[bank] > worst) worst = cnt[bank];
+      }
+    }
+    if (worst < best) { best = worst; best_pad = pad; }
+  }
+  t.C = C; t.HW = HW; t.gshift = gshift;
+  t.tiles = (HW + 4 * G - 1) / (4 * G);
+  t.pd = cd + best_pad;
+  t.aux = 4 * G * t.pd;
+  const unsigned long long m = ((1ull << 32) + cd - 1) / cd;
+  if (m >= (1ull << 32)) return false;
+  t.mg_cd = static_cast<unsigned>(m);
+  for (int v = 0; v < 4 * G * cd; ++v)
+    if (static_cast<int>((static_cast<unsigned long long>(v) * t.mg_cd) >> 32) != v / cd) return false;
+  *out = t;
+  *lds_bytes = bytes(gshift, t.pd);
+  return true;
+}
+
+struct NormVal { bool ok; NormTile t; size_t lds; };
+
+const NormVal& norm_tile_cached(int C, int HW, int esz) {
+  static thread_local std::unordered_map<TileKey, NormVal, TileKeyHash> cache;
+  const TileKey key = {C, HW, esz};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    if (cache.size() > 4096) cache.clear();
+    NormVal v = {};
+    v.ok = make_norm_tile(C, HW, static_cast<size_t>(esz), &v.t, &v.lds);
+    it = cache.emplace(key, v).first;
+  }
+  return it->second;
+}
+
 // float_tile: the caller can keep bf16 tensors as floats in LDS; taken where that still gives 64 pixels per tile.
 int check_block_args(const char* fn, int B, int C, int HW, int dtype, int pdtype, const TileVal** tv,
                      bool float_tile = false, int ntile = 1) {
@@ -107,6 +166,24 @@ extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight,
   const dim3 grid(tv->t.tiles, B);
   // rows of whole aligned 4-element vectors move as such
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0;
+  // rows of whole vectors: every value of a tile in a register of its own, where the channels fit
+  if (vec && (out_nhwc || reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0)) {
+    const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
+    if (nv.ok) {
+      auto launch_reg = [&](auto kern, auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (int e = allow_lds(kern, nv.lds)) return e;
+        WT_LAUNCH(kern, dim3(nv.t.tiles, B), dim3(kBlockThreads), nv.lds, stream, static_cast<const T*>(x),
+                  static_cast<T*>(out), weight, bias, param_dtype, eps, nv.t);
+        return check_launch("channel_norm_reg_kernel");
+      };
+      if (dtype == WTCONV_F32)
+        return out_nhwc ? launch_reg(channel_norm_reg_kernel<float, kNormPairs, true>, static_cast<float*>(nullptr))
+                        : launch_reg(channel_norm_reg_kernel<float, kNormPairs, false>, static_cast<float*>(nullptr));
+      return out_nhwc ? launch_reg(channel_norm_reg_kernel<bf16_t, kNormPairs, true>, static_cast<bf16_t*>(nullptr))
+                      : launch_reg(channel_norm_reg_kernel<bf16_t, kNormPairs, false>, static_cast<bf16_t*>(nullptr));
+    }
+  }
   auto launch = [&](auto kern, auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (int e = allow_lds(kern, tv->lds)) return e;
@@ -139,6 +216,20 @@ extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const 
   const dim3 grid(tv->t.tiles, B);
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(shortcut) % (4 * esz) == 0 &&
                    reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0;
+  if (vec) {
+    const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
+    if (nv.ok) {
+      auto launch_reg = [&](auto kern, auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (int e = allow_lds(kern, nv.lds)) return e;
+        WT_LAUNCH(kern, dim3(nv.t.tiles, B), dim3(kBlockThreads), nv.lds, stream, static_cast<const T*>(y),
+                  static_cast<const T*>(shortcut), gamma, param_dtype, static_cast<T*>(out), nv.t);
+        return check_launch("block_residual_reg_kernel");
+      };
+      return dtype == WTCONV_F32 ? launch_reg(block_residual_reg_kernel<float, kNormPairs>, static_cast<float*>(nullptr))
+                                 : launch_reg(block_residual_reg_kernel<bf16_t, kNormPairs>, static_cast<bf16_t*>(nullptr));
+    }
+  }
   auto launch = [&](auto kern, auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (int e = allow_lds(kern, tv->lds)) return e;

@@ -203,6 +203,182 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
   }
 }
 
+// ---- channel norm with the tile's values held in registers -----------------------------------------------------
+// For images whose rows move as 4-element vectors.  A workgroup takes `tp` = 4 G consecutive pixels (G a power of two,
+// 2..32) of one image; thread (g, e) = (tid % G, tid / G) owns pixels 4g..4g+3 of the channel pairs e, e + cs,
+// e + 2 cs, ... (cs = 256 / G, at most NP pairs): every value of the tile sits in one register of one thread from its
+// load to its store, the statistics are two exact passes over registers (mean, then squared deviations; partial sums
+// meet across the lanes of a wave that share g, then across the four waves through LDS), and LDS carries each
+// normalised value once, as the transpose to NHWC: a pixel-major tile [tp][pd dwords], written as packed channel
+// pairs and copied out as the one contiguous run it is in memory.  (NCHW output: no tile at all.)
+struct NormTile {
+  int C, HW;
+  int gshift;        // log2 G
+  int tiles;         // per image
+  int pd;            // dwords per pixel row of the LDS tile (C * sizeof(T) / 4 plus padding)
+  int aux;           // float index of the arrays behind the tile
+  unsigned mg_cd;    // reciprocal of the dwords per pixel (C * sizeof(T) / 4) for dividends below tp * that (shift 32)
+};
+
+template <typename T> struct PairWord;
+template <> struct PairWord<bf16_t> {
+  static constexpr int kDwords = 1;
+  static __device__ __forceinline__ void put(float* tile, int idx, float a, float b) {
+    reinterpret_cast<uint32_t*>(tile)[idx] = pack_bf16x2(a, b);
+  }
+};
+template <> struct PairWord<float> {
+  static constexpr int kDwords = 2;
+  static __device__ __forceinline__ void put(float* tile, int idx, float a, float b) { tile[idx] = a; tile[idx + 1] = b; }
+};
+
+template <typename T>
+__device__ __forceinline__ void store_quad(T* p, const float (&f)[4]);
+template <> __device__ __forceinline__ void store_quad<float>(float* p, const float (&f)[4]) {
+  float4 v;
+  v.x = f[0]; v.y = f[1]; v.z = f[2]; v.w = f[3];
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store_quad<bf16_t>(bf16_t* p, const float (&f)[4]) {
+  uint2 v;
+  v.x = pack_bf16x2(f[0], f[1]); v.y = pack_bf16x2(f[2], f[3]);
+  *reinterpret_cast<uint2*>(p) = v;
+}
+
+// Grid (tiles, B).  NHWC: out is (B, HW, C); else (B, C, HW).
+template <typename T, int NP, bool NHWC>
+__global__ void __launch_bounds__(kBlockThreads)
+channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __restrict__ weight,
+                        const void* __restrict__ bias, int pdtype, float eps, const NormTile t) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
+  const int g = tid & (G - 1), e = tid >> t.gshift;
+  const int C = t.C, C2 = C >> 1;
+  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
+  const bool live = 4 * g < np;                  // (HW % 4 == 0: a group of four pixels is inside the image or outside)
+  float* psum = ldsf + t.aux;                    // [4 waves][tp]
+  float* pvar = psum + 4 * tp;                   // [4 waves][tp]
+  float* wgt = pvar + 4 * tp;                    // weight[C], bias[C]
+  for (int c = tid; c < C; c += kBlockThreads) {
+    wgt[c] = load_param(weight, pdtype, c);
+    wgt[C + c] = load_param(bias, pdtype, c);
+  }
+  const T* src = x + static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
+  Quad<T> q[NP][2];
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      q[k][0].load(src + static_cast<size_t>(2 * cp) * t.HW);
+      q[k][1].load(src + static_cast<size_t>(2 * cp + 1) * t.HW);
+    }
+  }
+  float v[NP][2][4];
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    const bool on = live && cp < C2;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (on) q[k][h].get(v[k][h]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (!on) v[k][h][j] = 0.f;
+        s[j] += v[k][h][j];
+      }
+    }
+  }
+  // lanes of a wave that share g: lane bits gshift..5
+  const int lane4 = lane << 2;
+  auto meet = [&](float (&a)[4], float* part) {
+    for (int m = 32; m >= G; m >>= 1) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[j] += wave_xor(a[j], lane4, m);
+    }
+    if (lane < G) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[wave * tp + 4 * g + j] = a[j];
+    }
+  };
+  meet(s, psum);
+  __syncthreads();                               // (also: wgt is in place)
+  const float inv_c = 1.f / static_cast<float>(C);
+  float mean[4], sq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    mean[j] = (psum[4 * g + j] + psum[tp + 4 * g + j] + psum[2 * tp + 4 * g + j] + psum[3 * tp + 4 * g + j]) * inv_c;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const bool on = live && e + k * cs < C2;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float d = on ? v[k][h][j] - mean[j] : 0.f;
+        sq[j] += d * d;
+      }
+  }
+  meet(sq, pvar);
+  __syncthreads();
+  float rstd[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float var = (pvar[4 * g + j] + pvar[tp + 4 * g + j] + pvar[2 * tp + 4 * g + j] + pvar[3 * tp + 4 * g + j]) * inv_c;
+    rstd[j] = 1.f / sqrtf(var + eps);
+  }
+  constexpr int PW = PairWord<T>::kDwords;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      const int c = 2 * cp;
+      const float w0 = wgt[c], w1 = wgt[c + 1], b0 = wgt[C + c], b1 = wgt[C + c + 1];
+      float y0[4], y1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        y0[j] = (v[k][0][j] - mean[j]) * rstd[j] * w0 + b0;
+        y1[j] = (v[k][1][j] - mean[j]) * rstd[j] * w1 + b1;
+      }
+      if constexpr (NHWC) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) PairWord<T>::put(ldsf, (4 * g + j) * t.pd + cp * PW, y0[j], y1[j]);
+      } else {
+        T* dst = out + static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
+        store_quad<T>(dst + static_cast<size_t>(c) * t.HW, y0);
+        store_quad<T>(dst + static_cast<size_t>(c + 1) * t.HW, y1);
+      }
+    }
+  }
+  if constexpr (NHWC) {
+    __syncthreads();
+    // the tile's output is one contiguous run of np * C elements = np * cd dwords
+    const int cd = C2 * PW;
+    uint32_t* dst = reinterpret_cast<uint32_t*>(out + (static_cast<size_t>(b) * t.HW + p0) * C);
+    const uint32_t* tile = reinterpret_cast<const uint32_t*>(ldsf);
+    const int total = np * cd;
+    constexpr int kBatch = 8;                    // LDS reads a thread has under way before its stores
+    for (int i0 = tid; i0 < total; i0 += kBatch * kBlockThreads) {
+      uint32_t w[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int i = i0 + u * kBlockThreads;
+        if (i < total) {
+          const int pp = div_c(i, t.mg_cd);
+          w[u] = tile[pp * t.pd + (i - pp * cd)];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int i = i0 + u * kBlockThreads;
+        if (i < total) dst[i] = w[u];
+      }
+    }
+  }
+}
+
 // Grid (tiles, B).  y is (B, HW, C); shortcut and out are (B, C, HW); gamma may be null (no layer scale).
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
@@ -262,6 +438,91 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
         const size_t o = base + static_cast<size_t>(c) * t.HW;
         out[o] = from_f32<T>(to_f32<T>(shortcut[o]) + g * to_f32<T>(lds[c * pitch + p]));
       }
+    }
+  }
+}
+
+// The block's second pass on the plan of channel_norm_reg_kernel.  Grid (tiles, B).  The NHWC run of the tile goes into
+// LDS as it lies in memory (pixel-major, dword copies); thread (g, e) then takes the channel pairs e, e + cs, ... of
+// its four pixels from there as packed words, the shortcut's rows as 4-element vectors straight from HBM (issued before
+// the barrier), and writes the rows of the result.
+template <typename T> struct PairWordGet;
+template <> struct PairWordGet<bf16_t> {
+  static __device__ __forceinline__ void get(const float* tile, int idx, float& a, float& b) {
+    const uint32_t v = reinterpret_cast<const uint32_t*>(tile)[idx];
+    a = __uint_as_float(v << 16); b = __uint_as_float(v & 0xffff0000u);
+  }
+};
+template <> struct PairWordGet<float> {
+  static __device__ __forceinline__ void get(const float* tile, int idx, float& a, float& b) { a = tile[idx]; b = tile[idx + 1]; }
+};
+
+template <typename T, int NP>
+__global__ void __launch_bounds__(kBlockThreads)
+block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, const void* __restrict__ gamma,
+                          int pdtype, T* __restrict__ out, const NormTile t) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x;
+  const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
+  const int g = tid & (G - 1), e = tid >> t.gshift;
+  const int C = t.C, C2 = C >> 1;
+  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
+  const bool live = 4 * g < np;
+  constexpr int PW = PairWord<T>::kDwords;
+  const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
+  Quad<T> q[NP][2];
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      q[k][0].load(shortcut + base + static_cast<size_t>(2 * cp) * t.HW);
+      q[k][1].load(shortcut + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+    }
+  }
+  {
+    const int cd = C2 * PW;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + (static_cast<size_t>(b) * t.HW + p0) * C);
+    uint32_t* tile = reinterpret_cast<uint32_t*>(ldsf);
+    const int total = np * cd;
+    constexpr int kBatch = 8;                    // loads a thread keeps in flight
+    for (int i0 = tid; i0 < total; i0 += kBatch * kBlockThreads) {
+      uint32_t w[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int i = i0 + u * kBlockThreads;
+        if (i < total) w[u] = src[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int i = i0 + u * kBlockThreads;
+        if (i < total) {
+          const int pp = div_c(i, t.mg_cd);
+          tile[pp * t.pd + (i - pp * cd)] = w[u];
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      const int c = 2 * cp;
+      const float g0 = gamma != nullptr ? load_param(gamma, pdtype, c) : 1.f;
+      const float g1 = gamma != nullptr ? load_param(gamma, pdtype, c + 1) : 1.f;
+      float s0[4], s1[4];
+      q[k][0].get(s0);
+      q[k][1].get(s1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float a, bb;
+        PairWordGet<T>::get(ldsf, (4 * g + j) * t.pd + cp * PW, a, bb);
+        s0[j] += g0 * a;
+        s1[j] += g1 * bb;
+      }
+      store_quad<T>(out + base + static_cast<size_t>(c) * t.HW, s0);
+      store_quad<T>(out + base + static_cast<size_t>(c + 1) * t.HW, s1);
     }
   }
 }
