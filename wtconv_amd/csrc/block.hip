@@ -72,6 +72,10 @@ const TileVal& block_tile_cached(int C, int HW, int esz, int ntile = 1) {
 // holds at most `np_max` channel pairs; the padding of the pixel-major LDS tile that spreads a wave's writes best over
 // the banks.  false: too many channels for the registers of a workgroup (the LDS-tile kernel takes the call).
 constexpr int kNormPairs = 6;
+constexpr int kSumSlices = 32;        // slices of the two-stage column sum
+constexpr int kSumTickets = 64;       // its ticket words (column blocks of 64: up to 4096 columns)
+
+size_t block_record_floats(int B, int tiles, int C) { return (static_cast<size_t>(B) * tiles * 2 * C + 63) / 64 * 64; }
 
 bool make_norm_tile(int C, int HW, size_t esz, NormTile* out, size_t* lds_bytes) {
   const int C2 = C / 2, pw = static_cast<int>(esz) / 2;           // dwords per channel pair
@@ -252,8 +256,29 @@ extern "C" size_t wtconv_block_workspace_bytes(int B, int C, int HW, int dtype) 
   if (B <= 0 || C <= 0 || HW <= 0 || (dtype != WTCONV_F32 && dtype != WTCONV_BF16)) return 0;
   const TileVal& v = block_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2, 2);
   if (!v.ok) return 0;
-  const size_t bytes = static_cast<size_t>(B) * v.t.tiles * 2 * C * sizeof(float);
+  int tiles = v.t.tiles;                       // whichever plan a call takes: the larger record count
+  const NormVal& nv = norm_tile_cached(C, HW, dtype == WTCONV_F32 ? 4 : 2);
+  if (nv.ok && nv.t.tiles > tiles) tiles = nv.t.tiles;
+  // the records, then the slice sums and tickets of the two-stage column sum
+  const size_t bytes = (block_record_floats(B, tiles, C) + static_cast<size_t>(kSumSlices) * 2 * C) * sizeof(float) +
+                       kSumTickets * sizeof(unsigned);
   return (bytes + 255) / 256 * 256;
+}
+
+// Two-stage column sum of the register-plan kernels: slice sums and tickets behind the records (`rec_floats` of them;
+// the kernel that wrote the records has cleared the tickets).
+static unsigned* sum_tickets(float* partial, size_t rec_floats, int C) {
+  return reinterpret_cast<unsigned*>(partial + rec_floats + static_cast<size_t>(kSumSlices) * 2 * C);
+}
+
+static int launch_column_sum_sliced(float* partial, size_t rec_floats, int C, int nrec, int ncol, float* out0,
+                                    float* out1, int split, hipStream_t stream) {
+  int ns = nrec / 16;                          // at least 16 records per slice
+  if (ns > kSumSlices) ns = kSumSlices;
+  if (ns < 1) ns = 1;
+  WT_LAUNCH(column_sum_sliced_kernel, dim3((ncol + 63) / 64, ns), dim3(kBlockThreads), 0, stream, partial, nrec, ncol,
+            partial + rec_floats, sum_tickets(partial, rec_floats, C), out0, out1, split);
+  return check_launch("column_sum_sliced_kernel");
 }
 
 static int launch_column_sum(const float* partial, int nrec, int ncol, float* out0, float* out1, int split,
@@ -284,6 +309,30 @@ extern "C" int wtconv_channel_norm_backward(const void* x, const void* dy, const
                    reinterpret_cast<uintptr_t>(dx) % (4 * esz) == 0 &&
                    (dy_nhwc || reinterpret_cast<uintptr_t>(dy) % (4 * esz) == 0);
   float* partial = static_cast<float*>(workspace);
+  if (vec) {
+    const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
+    const size_t lds = nv.ok ? (static_cast<size_t>(nv.t.aux) + 16 * (4 << nv.t.gshift) + C) * sizeof(float) : 0;
+    if (nv.ok && lds <= 64 * 1024 && 2 * C <= 64 * kSumTickets) {
+      const size_t rec_floats = block_record_floats(B, nv.t.tiles, C);
+      auto launch_reg = [&](auto kern, auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (int e = allow_lds(kern, lds)) return e;
+        WT_LAUNCH(kern, dim3(nv.t.tiles, B), dim3(kBlockThreads), lds, stream, static_cast<const T*>(x),
+                  static_cast<const T*>(dy), weight, param_dtype, eps, static_cast<T*>(dx), partial, nv.t,
+                  sum_tickets(partial, rec_floats, C), kSumTickets);
+        return check_launch("channel_norm_bwd_reg_kernel");
+      };
+      int e;
+      if (dtype == WTCONV_F32)
+        e = dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<float, kNormPairs, true>, static_cast<float*>(nullptr))
+                    : launch_reg(channel_norm_bwd_reg_kernel<float, kNormPairs, false>, static_cast<float*>(nullptr));
+      else
+        e = dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<bf16_t, kNormPairs, true>, static_cast<bf16_t*>(nullptr))
+                    : launch_reg(channel_norm_bwd_reg_kernel<bf16_t, kNormPairs, false>, static_cast<bf16_t*>(nullptr));
+      if (e) return e;
+      return launch_column_sum_sliced(partial, rec_floats, C, B * nv.t.tiles, 2 * C, dweight, dbias, C, stream);
+    }
+  }
   auto launch = [&](auto kern, auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (int e = allow_lds(kern, tv->lds)) return e;
@@ -321,6 +370,25 @@ extern "C" int wtconv_block_residual_backward(const void* dout, const void* y, c
   const dim3 grid(tv->t.tiles, B);
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(dout) % (4 * esz) == 0;
   float* partial = static_cast<float*>(workspace);
+  if (vec) {
+    const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
+    if (nv.ok && C <= 64 * kSumTickets) {
+      const size_t rec_floats = block_record_floats(B, nv.t.tiles, C);
+      auto launch_reg = [&](auto kern, auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (int e = allow_lds(kern, nv.lds)) return e;
+        WT_LAUNCH(kern, dim3(nv.t.tiles, B), dim3(kBlockThreads), nv.lds, stream, static_cast<const T*>(dout),
+                  static_cast<const T*>(y), gamma, param_dtype, static_cast<T*>(dy), partial, nv.t,
+                  sum_tickets(partial, rec_floats, C), kSumTickets);
+        return check_launch("block_residual_bwd_reg_kernel");
+      };
+      const int e = dtype == WTCONV_F32
+                        ? launch_reg(block_residual_bwd_reg_kernel<float, kNormPairs>, static_cast<float*>(nullptr))
+                        : launch_reg(block_residual_bwd_reg_kernel<bf16_t, kNormPairs>, static_cast<bf16_t*>(nullptr));
+      if (e) return e;
+      return launch_column_sum_sliced(partial, rec_floats, C, B * nv.t.tiles, C, dgamma, dgamma, C, stream);
+    }
+  }
   auto launch = [&](auto kern, auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     if (int e = allow_lds(kern, tv->lds)) return e;

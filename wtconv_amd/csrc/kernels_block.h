@@ -693,6 +693,294 @@ block_residual_bwd_kernel(const T* __restrict__ dout, const T* __restrict__ y, c
   }
 }
 
+// ---- backward passes on the plan of channel_norm_reg_kernel (rows of whole 4-element vectors) ---------------------------
+// Sum of `v` over the G = 2^gshift lanes that differ in their low lane bits (the pixel groups of one channel pair);
+// every lane of the group gets the total.  DPP within rows of 16 lanes, one cross-lane exchange for G = 32.
+__device__ __forceinline__ float group_sum(float v, int gshift, int lane4) {
+#ifdef WT_EMULATE
+  (void)lane4;
+  for (int m = 1; m < (1 << gshift); m <<= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+#else
+  auto dpp = [](float x, auto ctrl) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value, 0xf, 0xf, false));
+  };
+  using std::integral_constant;
+  if (gshift >= 1) v += dpp(v, integral_constant<int, 0xB1>{});     // quad_perm [1,0,3,2]
+  if (gshift >= 2) v += dpp(v, integral_constant<int, 0x4E>{});     // quad_perm [2,3,0,1]
+  if (gshift >= 3) v += dpp(v, integral_constant<int, 0x141>{});    // row_half_mirror
+  if (gshift >= 4) v += dpp(v, integral_constant<int, 0x140>{});    // row_mirror
+  if (gshift >= 5) v += wave_xor(v, lane4, 16);
+  return v;
+#endif
+}
+
+// A contiguous run of `total` dwords -> the pixel-major LDS tile (rows of cd dwords at a pitch of pd), eight loads in
+// flight per thread; and back.
+__device__ __forceinline__ void tile_from_run(const uint32_t* __restrict__ src, uint32_t* tile, int total, int cd,
+                                              const NormTile& t, int tid) {
+  constexpr int kBatch = 8;
+  for (int i0 = tid; i0 < total; i0 += kBatch * kBlockThreads) {
+    uint32_t w[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = i0 + u * kBlockThreads;
+      if (i < total) w[u] = src[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = i0 + u * kBlockThreads;
+      if (i < total) {
+        const int pp = div_c(i, t.mg_cd);
+        tile[pp * t.pd + (i - pp * cd)] = w[u];
+      }
+    }
+  }
+}
+__device__ __forceinline__ void tile_to_run(const uint32_t* tile, uint32_t* __restrict__ dst, int total, int cd,
+                                            const NormTile& t, int tid) {
+  constexpr int kBatch = 8;
+  for (int i0 = tid; i0 < total; i0 += kBatch * kBlockThreads) {
+    uint32_t w[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = i0 + u * kBlockThreads;
+      if (i < total) {
+        const int pp = div_c(i, t.mg_cd);
+        w[u] = tile[pp * t.pd + (i - pp * cd)];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = i0 + u * kBlockThreads;
+      if (i < total) dst[i] = w[u];
+    }
+  }
+}
+
+// Backward of the channel norm, values in registers.  Grid (tiles, B); arguments as channel_norm_bwd_kernel.  The
+// gradient arrives as rows (NCHW: straight into registers) or as the tile's contiguous NHWC run (through the LDS tile,
+// read back as packed channel pairs).  Four sums per pixel (x, squared deviations, g, g * xh) meet as in the forward
+// kernel; the per-channel sums over the tile's pixels meet across the pixel groups with group_sum.
+template <typename T, int NP, bool DY_NHWC>
+__global__ void __launch_bounds__(kBlockThreads)
+channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, const void* __restrict__ weight,
+                            int pdtype, float eps, T* __restrict__ dx, float* __restrict__ partial, const NormTile t,
+                            unsigned* __restrict__ zero_words, int nzero) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (blockIdx.x == 0 && blockIdx.y == 0)        // the tickets of the column sum that follows on the stream
+    for (int i = tid; i < nzero; i += kBlockThreads) zero_words[i] = 0u;
+  const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
+  const int g = tid & (G - 1), e = tid >> t.gshift;
+  const int C = t.C, C2 = C >> 1;
+  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
+  const bool live = 4 * g < np;
+  constexpr int PW = PairWord<T>::kDwords;
+  float* part = ldsf + t.aux;                    // four arrays [4 waves][tp]
+  float* wgt = part + 16 * tp;                   // weight[C]
+  for (int c = tid; c < C; c += kBlockThreads) wgt[c] = load_param(weight, pdtype, c);
+  const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
+  Quad<T> q[NP][2];
+  Quad<T> qd[DY_NHWC ? 1 : NP][2];
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      q[k][0].load(x + base + static_cast<size_t>(2 * cp) * t.HW);
+      q[k][1].load(x + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+      if constexpr (!DY_NHWC) {
+        qd[k][0].load(dy + base + static_cast<size_t>(2 * cp) * t.HW);
+        qd[k][1].load(dy + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+      }
+    }
+  }
+  const int cd = C2 * PW;
+  if constexpr (DY_NHWC)
+    tile_from_run(reinterpret_cast<const uint32_t*>(dy + (static_cast<size_t>(b) * t.HW + p0) * C),
+                  reinterpret_cast<uint32_t*>(ldsf), np * cd, cd, t, tid);
+  float v[NP][2][4];
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const bool on = live && e + k * cs < C2;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (on) q[k][h].get(v[k][h]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (!on) v[k][h][j] = 0.f;
+        s[j] += v[k][h][j];
+      }
+    }
+  }
+  const int lane4 = lane << 2;
+  auto meet = [&](float (&a)[4], float* arr) {
+    for (int m = 32; m >= G; m >>= 1) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[j] += wave_xor(a[j], lane4, m);
+    }
+    if (lane < G) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) arr[wave * tp + 4 * g + j] = a[j];
+    }
+  };
+  auto total = [&](const float* arr, int j) {
+    return arr[4 * g + j] + arr[tp + 4 * g + j] + arr[2 * tp + 4 * g + j] + arr[3 * tp + 4 * g + j];
+  };
+  meet(s, part);
+  __syncthreads();                               // (also: the weights and the gradient tile are in place)
+  const float inv_c = 1.f / static_cast<float>(C);
+  float mean[4], sq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) mean[j] = total(part, j) * inv_c;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const bool on = live && e + k * cs < C2;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float d = on ? v[k][h][j] - mean[j] : 0.f;
+        v[k][h][j] = d;                          // from here on: deviations
+        sq[j] += d * d;
+      }
+  }
+  meet(sq, part + 4 * tp);
+  __syncthreads();
+  float rstd[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rstd[j] = 1.f / sqrtf(total(part + 4 * tp, j) * inv_c + eps);
+  // the gradient of this thread's values: (d0, d1) of pixel j, channel pair k
+  auto grad_pair = [&](int k, int j, float& d0, float& d1) {
+    if constexpr (DY_NHWC) {
+      PairWordGet<T>::get(ldsf, (4 * g + j) * t.pd + (e + k * cs) * PW, d0, d1);
+    } else {
+      float f0[4], f1[4];
+      qd[k][0].get(f0);
+      qd[k][1].get(f1);
+      d0 = f0[j]; d1 = f1[j];
+    }
+  };
+  float a1[4] = {0.f, 0.f, 0.f, 0.f}, a2[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      const float w0 = wgt[2 * cp], w1 = wgt[2 * cp + 1];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float d0, d1;
+        grad_pair(k, j, d0, d1);
+        const float g0 = d0 * w0, g1 = d1 * w1;
+        a1[j] += g0 + g1;
+        a2[j] += (g0 * v[k][0][j] + g1 * v[k][1][j]) * rstd[j];
+      }
+    }
+  }
+  meet(a1, part + 8 * tp);
+  meet(a2, part + 12 * tp);
+  __syncthreads();
+  float m1[4], m2[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    m1[j] = total(part + 8 * tp, j) * inv_c;
+    m2[j] = total(part + 12 * tp, j) * inv_c;
+  }
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * 2 * C;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    const bool on = live && cp < C2;
+    float dw0 = 0.f, dw1 = 0.f, db0 = 0.f, db1 = 0.f;
+    if (on) {
+      const float w0 = wgt[2 * cp], w1 = wgt[2 * cp + 1];
+      float o0[4], o1[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float d0, d1;
+        grad_pair(k, j, d0, d1);
+        const float xh0 = v[k][0][j] * rstd[j], xh1 = v[k][1][j] * rstd[j];
+        o0[j] = rstd[j] * (d0 * w0 - m1[j] - xh0 * m2[j]);
+        o1[j] = rstd[j] * (d1 * w1 - m1[j] - xh1 * m2[j]);
+        dw0 += d0 * xh0; dw1 += d1 * xh1;
+        db0 += d0; db1 += d1;
+      }
+      store_quad<T>(dx + base + static_cast<size_t>(2 * cp) * t.HW, o0);
+      store_quad<T>(dx + base + static_cast<size_t>(2 * cp + 1) * t.HW, o1);
+    }
+    dw0 = group_sum(dw0, t.gshift, lane4); dw1 = group_sum(dw1, t.gshift, lane4);
+    db0 = group_sum(db0, t.gshift, lane4); db1 = group_sum(db1, t.gshift, lane4);
+    if (g == 0 && cp < C2) {
+      rec[2 * cp] = dw0; rec[2 * cp + 1] = dw1;
+      rec[C + 2 * cp] = db0; rec[C + 2 * cp + 1] = db1;
+    }
+  }
+}
+
+// Backward of the block residual on the same plan.  Grid (tiles, B); arguments as block_residual_bwd_kernel.  The NHWC
+// run of y goes through the LDS tile; each thread replaces the words it reads there by gamma * dout, and the tile leaves
+// as the contiguous run of dy.
+template <typename T, int NP>
+__global__ void __launch_bounds__(kBlockThreads)
+block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ y, const void* __restrict__ gamma,
+                              int pdtype, T* __restrict__ dy, float* __restrict__ partial, const NormTile t,
+                              unsigned* __restrict__ zero_words, int nzero) {
+  WT_SHARED_FLOATS(ldsf);
+  const int tid = threadIdx.x, lane = tid & 63;
+  if (blockIdx.x == 0 && blockIdx.y == 0)        // the tickets of the column sum that follows on the stream
+    for (int i = tid; i < nzero; i += kBlockThreads) zero_words[i] = 0u;
+  const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
+  const int g = tid & (G - 1), e = tid >> t.gshift;
+  const int C = t.C, C2 = C >> 1;
+  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
+  const bool live = 4 * g < np;
+  constexpr int PW = PairWord<T>::kDwords;
+  const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
+  Quad<T> q[NP][2];
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    if (live && cp < C2) {
+      q[k][0].load(dout + base + static_cast<size_t>(2 * cp) * t.HW);
+      q[k][1].load(dout + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+    }
+  }
+  const int cd = C2 * PW;
+  const size_t run = (static_cast<size_t>(b) * t.HW + p0) * C;
+  tile_from_run(reinterpret_cast<const uint32_t*>(y + run), reinterpret_cast<uint32_t*>(ldsf), np * cd, cd, t, tid);
+  __syncthreads();
+  const int lane4 = lane << 2;
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * C;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int cp = e + k * cs;
+    float dg0 = 0.f, dg1 = 0.f;
+    if (live && cp < C2) {
+      const float g0 = load_param(gamma, pdtype, 2 * cp), g1 = load_param(gamma, pdtype, 2 * cp + 1);
+      float d0[4], d1[4];
+      q[k][0].get(d0);
+      q[k][1].get(d1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = (4 * g + j) * t.pd + cp * PW;
+        float ya, yb;
+        PairWordGet<T>::get(ldsf, idx, ya, yb);
+        dg0 += d0[j] * ya;
+        dg1 += d1[j] * yb;
+        PairWord<T>::put(ldsf, idx, g0 * d0[j], g1 * d1[j]);
+      }
+    }
+    dg0 = group_sum(dg0, t.gshift, lane4);
+    dg1 = group_sum(dg1, t.gshift, lane4);
+    if (g == 0 && cp < C2) { rec[2 * cp] = dg0; rec[2 * cp + 1] = dg1; }
+  }
+  __syncthreads();
+  tile_to_run(reinterpret_cast<const uint32_t*>(ldsf), reinterpret_cast<uint32_t*>(dy + run), np * cd, cd, t, tid);
+}
+
 // out[v] = sum over the `nrec` records of partial[r][v], v < ncol, added in record order (grid = ceil(ncol / 64)
 // workgroups of 256 threads: four row groups per column, joined through LDS in a fixed order).
 __global__ void __launch_bounds__(kBlockThreads) column_sum_kernel(const float* __restrict__ partial, int nrec, int ncol,
@@ -713,6 +1001,49 @@ __global__ void __launch_bounds__(kBlockThreads) column_sum_kernel(const float* 
     const float v = (red[threadIdx.x] + red[threadIdx.x + 64]) + (red[threadIdx.x + 128] + red[threadIdx.x + 192]);
     if (col < split) out0[col] = v;
     else out1[col - split] = v;
+  }
+}
+
+// The same sum for many records, in two fixed stages inside one launch.  Grid (ceil(ncol / 64), ns): workgroup
+// (cb, s) sums the records of slice s (contiguous, ceil(nrec / ns) of them) for its 64 columns and leaves the result in
+// slices[s][col]; the workgroup of a column block that finishes last adds the ns slice sums in slice order.  `tickets`:
+// one zeroed word per column block (left zero again).
+__global__ void __launch_bounds__(kBlockThreads)
+column_sum_sliced_kernel(const float* __restrict__ partial, int nrec, int ncol, float* __restrict__ slices,
+                         unsigned* __restrict__ tickets, float* __restrict__ out0, float* __restrict__ out1, int split) {
+  __shared__ float red[kBlockThreads];
+  __shared__ unsigned flag;
+  const int col = blockIdx.x * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
+  const int ns = gridDim.y, sl = blockIdx.y;
+  const int per = (nrec + ns - 1) / ns;
+  const int rb = sl * per, re = rb + per < nrec ? rb + per : nrec;
+  float s = 0.f;
+  if (col < ncol && rb < re) {
+    const int per_g = (re - rb + 3) / 4;
+    const int r0 = rb + grp * per_g, r1 = r0 + per_g < re ? r0 + per_g : re;
+#pragma unroll 8
+    for (int r = r0; r < r1; ++r) s += partial[static_cast<size_t>(r) * ncol + col];
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  if (grp == 0 && col < ncol) {
+    const float v = (red[threadIdx.x] + red[threadIdx.x + 64]) + (red[threadIdx.x + 128] + red[threadIdx.x + 192]);
+    store_shared_f32(slices + static_cast<size_t>(sl) * ncol + col, v);
+  }
+  if (workgroup_is_last(tickets + blockIdx.x, static_cast<unsigned>(ns), &flag)) {
+    if (grp == 0 && col < ncol) {
+      float v = 0.f;
+      for (int q0 = 0; q0 < ns; q0 += 8) {       // eight loads under way, added in slice order
+        float w[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) w[u] = q0 + u < ns ? load_shared_f32(slices + static_cast<size_t>(q0 + u) * ncol + col) : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += w[u];
+      }
+      if (col < split) out0[col] = v;
+      else out1[col - split] = v;
+    }
+    if (threadIdx.x == 0) tickets[blockIdx.x] = 0u;
   }
 }
 
