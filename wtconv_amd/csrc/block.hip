@@ -170,10 +170,12 @@ extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight,
   const dim3 grid(tv->t.tiles, B);
   // rows of whole aligned 4-element vectors move as such
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0;
-  // rows of whole vectors: every value of a tile in a register of its own, where the channels fit
-  if (vec && (out_nhwc || reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0)) {
+  // every value of a tile in a register of its own, where the channels fit
+  {
+    // (rows that move element by element: measured no faster than the LDS-tile kernel below, which keeps them)
+    const bool v4 = vec && (out_nhwc || reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0);
     const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
-    if (nv.ok) {
+    if (nv.ok && v4) {
       auto launch_reg = [&](auto kern, auto* tag) {
         using T = std::remove_pointer_t<decltype(tag)>;
         if (int e = allow_lds(kern, nv.lds)) return e;
@@ -181,11 +183,14 @@ extern "C" int wtconv_channel_norm(const void* x, void* out, const void* weight,
                   static_cast<T*>(out), weight, bias, param_dtype, eps, nv.t);
         return check_launch("channel_norm_reg_kernel");
       };
-      if (dtype == WTCONV_F32)
-        return out_nhwc ? launch_reg(channel_norm_reg_kernel<float, kNormPairs, true>, static_cast<float*>(nullptr))
-                        : launch_reg(channel_norm_reg_kernel<float, kNormPairs, false>, static_cast<float*>(nullptr));
-      return out_nhwc ? launch_reg(channel_norm_reg_kernel<bf16_t, kNormPairs, true>, static_cast<bf16_t*>(nullptr))
-                      : launch_reg(channel_norm_reg_kernel<bf16_t, kNormPairs, false>, static_cast<bf16_t*>(nullptr));
+      auto by_layout = [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (v4) return out_nhwc ? launch_reg(channel_norm_reg_kernel<T, kNormPairs, true, true>, tag)
+                                : launch_reg(channel_norm_reg_kernel<T, kNormPairs, false, true>, tag);
+        return out_nhwc ? launch_reg(channel_norm_reg_kernel<T, kNormPairs, true, false>, tag)
+                        : launch_reg(channel_norm_reg_kernel<T, kNormPairs, false, false>, tag);
+      };
+      return dtype == WTCONV_F32 ? by_layout(static_cast<float*>(nullptr)) : by_layout(static_cast<bf16_t*>(nullptr));
     }
   }
   auto launch = [&](auto kern, auto* tag) {
@@ -220,9 +225,9 @@ extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const 
   const dim3 grid(tv->t.tiles, B);
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(shortcut) % (4 * esz) == 0 &&
                    reinterpret_cast<uintptr_t>(out) % (4 * esz) == 0;
-  if (vec) {
+  {
     const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
-    if (nv.ok) {
+    if (nv.ok && vec) {      // (element-wise rows: the LDS-tile kernel below measured faster)
       auto launch_reg = [&](auto kern, auto* tag) {
         using T = std::remove_pointer_t<decltype(tag)>;
         if (int e = allow_lds(kern, nv.lds)) return e;
@@ -230,8 +235,12 @@ extern "C" int wtconv_block_residual(const void* y, const void* shortcut, const 
                   static_cast<const T*>(shortcut), gamma, param_dtype, static_cast<T*>(out), nv.t);
         return check_launch("block_residual_reg_kernel");
       };
-      return dtype == WTCONV_F32 ? launch_reg(block_residual_reg_kernel<float, kNormPairs>, static_cast<float*>(nullptr))
-                                 : launch_reg(block_residual_reg_kernel<bf16_t, kNormPairs>, static_cast<bf16_t*>(nullptr));
+      auto by_rows = [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        return vec ? launch_reg(block_residual_reg_kernel<T, kNormPairs, true>, tag)
+                   : launch_reg(block_residual_reg_kernel<T, kNormPairs, false>, tag);
+      };
+      return dtype == WTCONV_F32 ? by_rows(static_cast<float*>(nullptr)) : by_rows(static_cast<bf16_t*>(nullptr));
     }
   }
   auto launch = [&](auto kern, auto* tag) {
@@ -309,7 +318,7 @@ extern "C" int wtconv_channel_norm_backward(const void* x, const void* dy, const
                    reinterpret_cast<uintptr_t>(dx) % (4 * esz) == 0 &&
                    (dy_nhwc || reinterpret_cast<uintptr_t>(dy) % (4 * esz) == 0);
   float* partial = static_cast<float*>(workspace);
-  if (vec) {
+  {
     const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
     const size_t lds = nv.ok ? (static_cast<size_t>(nv.t.aux) + 16 * (4 << nv.t.gshift) + C) * sizeof(float) : 0;
     if (nv.ok && lds <= 64 * 1024 && 2 * C <= 64 * kSumTickets) {
@@ -322,13 +331,14 @@ extern "C" int wtconv_channel_norm_backward(const void* x, const void* dy, const
                   sum_tickets(partial, rec_floats, C), kSumTickets);
         return check_launch("channel_norm_bwd_reg_kernel");
       };
-      int e;
-      if (dtype == WTCONV_F32)
-        e = dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<float, kNormPairs, true>, static_cast<float*>(nullptr))
-                    : launch_reg(channel_norm_bwd_reg_kernel<float, kNormPairs, false>, static_cast<float*>(nullptr));
-      else
-        e = dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<bf16_t, kNormPairs, true>, static_cast<bf16_t*>(nullptr))
-                    : launch_reg(channel_norm_bwd_reg_kernel<bf16_t, kNormPairs, false>, static_cast<bf16_t*>(nullptr));
+      auto by_layout = [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (vec) return dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<T, kNormPairs, true, true>, tag)
+                                : launch_reg(channel_norm_bwd_reg_kernel<T, kNormPairs, false, true>, tag);
+        return dy_nhwc ? launch_reg(channel_norm_bwd_reg_kernel<T, kNormPairs, true, false>, tag)
+                       : launch_reg(channel_norm_bwd_reg_kernel<T, kNormPairs, false, false>, tag);
+      };
+      const int e = dtype == WTCONV_F32 ? by_layout(static_cast<float*>(nullptr)) : by_layout(static_cast<bf16_t*>(nullptr));
       if (e) return e;
       return launch_column_sum_sliced(partial, rec_floats, C, B * nv.t.tiles, 2 * C, dweight, dbias, C, stream);
     }
@@ -370,7 +380,7 @@ extern "C" int wtconv_block_residual_backward(const void* dout, const void* y, c
   const dim3 grid(tv->t.tiles, B);
   const bool vec = HW % 4 == 0 && reinterpret_cast<uintptr_t>(dout) % (4 * esz) == 0;
   float* partial = static_cast<float*>(workspace);
-  if (vec) {
+  {
     const NormVal& nv = norm_tile_cached(C, HW, static_cast<int>(esz));
     if (nv.ok && C <= 64 * kSumTickets) {
       const size_t rec_floats = block_record_floats(B, nv.t.tiles, C);
@@ -382,9 +392,12 @@ extern "C" int wtconv_block_residual_backward(const void* dout, const void* y, c
                   sum_tickets(partial, rec_floats, C), kSumTickets);
         return check_launch("block_residual_bwd_reg_kernel");
       };
-      const int e = dtype == WTCONV_F32
-                        ? launch_reg(block_residual_bwd_reg_kernel<float, kNormPairs>, static_cast<float*>(nullptr))
-                        : launch_reg(block_residual_bwd_reg_kernel<bf16_t, kNormPairs>, static_cast<bf16_t*>(nullptr));
+      auto by_rows = [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        return vec ? launch_reg(block_residual_bwd_reg_kernel<T, kNormPairs, true>, tag)
+                   : launch_reg(block_residual_bwd_reg_kernel<T, kNormPairs, false>, tag);
+      };
+      const int e = dtype == WTCONV_F32 ? by_rows(static_cast<float*>(nullptr)) : by_rows(static_cast<bf16_t*>(nullptr));
       if (e) return e;
       return launch_column_sum_sliced(partial, rec_floats, C, B * nv.t.tiles, C, dgamma, dgamma, C, stream);
     }

@@ -74,12 +74,20 @@ template <typename T> struct Quad;
 template <> struct Quad<float> {
   float4 v;
   __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
+  // the first n of four elements one by one (any alignment), the rest zero
+  __device__ __forceinline__ void load_n(const float* p, int n) {
+    v.x = n > 0 ? p[0] : 0.f; v.y = n > 1 ? p[1] : 0.f; v.z = n > 2 ? p[2] : 0.f; v.w = n > 3 ? p[3] : 0.f;
+  }
   __device__ __forceinline__ void get(float (&f)[4]) const { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
   __device__ __forceinline__ void raw(float (&f)[4]) const { get(f); }
 };
 template <> struct Quad<bf16_t> {
   uint2 v;
   __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const uint2*>(p); }
+  __device__ __forceinline__ void load_n(const bf16_t* p, int n) {
+    const uint32_t a = n > 0 ? p[0] : 0u, b = n > 1 ? p[1] : 0u, c = n > 2 ? p[2] : 0u, d = n > 3 ? p[3] : 0u;
+    v.x = a | (b << 16); v.y = c | (d << 16);
+  }
   __device__ __forceinline__ void get(float (&f)[4]) const {
     f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
     f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
@@ -204,7 +212,7 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
 }
 
 // ---- channel norm with the tile's values held in registers -----------------------------------------------------
-// For images whose rows move as 4-element vectors.  A workgroup takes `tp` = 4 G consecutive pixels (G a power of two,
+// Rows move as 4-element vectors (VEC: HW a multiple of 4, aligned tensors) or element by element.  A workgroup takes `tp` = 4 G consecutive pixels (G a power of two,
 // 2..32) of one image; thread (g, e) = (tid % G, tid / G) owns pixels 4g..4g+3 of the channel pairs e, e + cs,
 // e + 2 cs, ... (cs = 256 / G, at most NP pairs): every value of the tile sits in one register of one thread from its
 // load to its store, the statistics are two exact passes over registers (mean, then squared deviations; partial sums
@@ -244,9 +252,25 @@ template <> __device__ __forceinline__ void store_quad<bf16_t>(bf16_t* p, const 
   v.x = pack_bf16x2(f[0], f[1]); v.y = pack_bf16x2(f[2], f[3]);
   *reinterpret_cast<uint2*>(p) = v;
 }
+// VEC: four elements as one aligned vector; else the first n one by one.
+template <typename T, bool VEC>
+__device__ __forceinline__ void load_row4(Quad<T>& q, const T* p, int n) {
+  if constexpr (VEC) q.load(p);
+  else q.load_n(p, n);
+}
+template <typename T, bool VEC>
+__device__ __forceinline__ void store_row4(T* p, const float (&f)[4], int n) {
+  if constexpr (VEC) {
+    store_quad<T>(p, f);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < n) p[j] = from_f32<T>(f[j]);
+  }
+}
 
 // Grid (tiles, B).  NHWC: out is (B, HW, C); else (B, C, HW).
-template <typename T, int NP, bool NHWC>
+template <typename T, int NP, bool NHWC, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __restrict__ weight,
                         const void* __restrict__ bias, int pdtype, float eps, const NormTile t) {
@@ -257,7 +281,8 @@ channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void
   const int C = t.C, C2 = C >> 1;
   const int p0 = blockIdx.x * tp, b = blockIdx.y;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
-  const bool live = 4 * g < np;                  // (HW % 4 == 0: a group of four pixels is inside the image or outside)
+  const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
+  const bool live = nv > 0;
   float* psum = ldsf + t.aux;                    // [4 waves][tp]
   float* pvar = psum + 4 * tp;                   // [4 waves][tp]
   float* wgt = pvar + 4 * tp;                    // weight[C], bias[C]
@@ -271,8 +296,8 @@ channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
     if (live && cp < C2) {
-      q[k][0].load(src + static_cast<size_t>(2 * cp) * t.HW);
-      q[k][1].load(src + static_cast<size_t>(2 * cp + 1) * t.HW);
+      load_row4<T, VEC>(q[k][0], src + static_cast<size_t>(2 * cp) * t.HW, nv);
+      load_row4<T, VEC>(q[k][1], src + static_cast<size_t>(2 * cp + 1) * t.HW, nv);
     }
   }
   float v[NP][2][4];
@@ -347,8 +372,8 @@ channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void
         for (int j = 0; j < 4; ++j) PairWord<T>::put(ldsf, (4 * g + j) * t.pd + cp * PW, y0[j], y1[j]);
       } else {
         T* dst = out + static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
-        store_quad<T>(dst + static_cast<size_t>(c) * t.HW, y0);
-        store_quad<T>(dst + static_cast<size_t>(c + 1) * t.HW, y1);
+        store_row4<T, VEC>(dst + static_cast<size_t>(c) * t.HW, y0, nv);
+        store_row4<T, VEC>(dst + static_cast<size_t>(c + 1) * t.HW, y1, nv);
       }
     }
   }
@@ -457,7 +482,7 @@ template <> struct PairWordGet<float> {
   static __device__ __forceinline__ void get(const float* tile, int idx, float& a, float& b) { a = tile[idx]; b = tile[idx + 1]; }
 };
 
-template <typename T, int NP>
+template <typename T, int NP, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, const void* __restrict__ gamma,
                           int pdtype, T* __restrict__ out, const NormTile t) {
@@ -468,7 +493,8 @@ block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcu
   const int C = t.C, C2 = C >> 1;
   const int p0 = blockIdx.x * tp, b = blockIdx.y;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
-  const bool live = 4 * g < np;
+  const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
+  const bool live = nv > 0;
   constexpr int PW = PairWord<T>::kDwords;
   const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
   Quad<T> q[NP][2];
@@ -476,8 +502,8 @@ block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcu
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
     if (live && cp < C2) {
-      q[k][0].load(shortcut + base + static_cast<size_t>(2 * cp) * t.HW);
-      q[k][1].load(shortcut + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+      load_row4<T, VEC>(q[k][0], shortcut + base + static_cast<size_t>(2 * cp) * t.HW, nv);
+      load_row4<T, VEC>(q[k][1], shortcut + base + static_cast<size_t>(2 * cp + 1) * t.HW, nv);
     }
   }
   {
@@ -516,13 +542,15 @@ block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcu
       q[k][1].get(s1);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float a, bb;
-        PairWordGet<T>::get(ldsf, (4 * g + j) * t.pd + cp * PW, a, bb);
-        s0[j] += g0 * a;
-        s1[j] += g1 * bb;
+        if (VEC || j < nv) {
+          float a, bb;
+          PairWordGet<T>::get(ldsf, (4 * g + j) * t.pd + cp * PW, a, bb);
+          s0[j] += g0 * a;
+          s1[j] += g1 * bb;
+        }
       }
-      store_quad<T>(out + base + static_cast<size_t>(c) * t.HW, s0);
-      store_quad<T>(out + base + static_cast<size_t>(c + 1) * t.HW, s1);
+      store_row4<T, VEC>(out + base + static_cast<size_t>(c) * t.HW, s0, nv);
+      store_row4<T, VEC>(out + base + static_cast<size_t>(c + 1) * t.HW, s1, nv);
     }
   }
 }
@@ -762,7 +790,7 @@ __device__ __forceinline__ void tile_to_run(const uint32_t* tile, uint32_t* __re
 // gradient arrives as rows (NCHW: straight into registers) or as the tile's contiguous NHWC run (through the LDS tile,
 // read back as packed channel pairs).  Four sums per pixel (x, squared deviations, g, g * xh) meet as in the forward
 // kernel; the per-channel sums over the tile's pixels meet across the pixel groups with group_sum.
-template <typename T, int NP, bool DY_NHWC>
+template <typename T, int NP, bool DY_NHWC, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, const void* __restrict__ weight,
                             int pdtype, float eps, T* __restrict__ dx, float* __restrict__ partial, const NormTile t,
@@ -776,7 +804,8 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
   const int C = t.C, C2 = C >> 1;
   const int p0 = blockIdx.x * tp, b = blockIdx.y;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
-  const bool live = 4 * g < np;
+  const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
+  const bool live = nv > 0;
   constexpr int PW = PairWord<T>::kDwords;
   float* part = ldsf + t.aux;                    // four arrays [4 waves][tp]
   float* wgt = part + 16 * tp;                   // weight[C]
@@ -788,11 +817,11 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
     if (live && cp < C2) {
-      q[k][0].load(x + base + static_cast<size_t>(2 * cp) * t.HW);
-      q[k][1].load(x + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+      load_row4<T, VEC>(q[k][0], x + base + static_cast<size_t>(2 * cp) * t.HW, nv);
+      load_row4<T, VEC>(q[k][1], x + base + static_cast<size_t>(2 * cp + 1) * t.HW, nv);
       if constexpr (!DY_NHWC) {
-        qd[k][0].load(dy + base + static_cast<size_t>(2 * cp) * t.HW);
-        qd[k][1].load(dy + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+        load_row4<T, VEC>(qd[k][0], dy + base + static_cast<size_t>(2 * cp) * t.HW, nv);
+        load_row4<T, VEC>(qd[k][1], dy + base + static_cast<size_t>(2 * cp + 1) * t.HW, nv);
       }
     }
   }
@@ -871,11 +900,13 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
       const float w0 = wgt[2 * cp], w1 = wgt[2 * cp + 1];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float d0, d1;
-        grad_pair(k, j, d0, d1);
-        const float g0 = d0 * w0, g1 = d1 * w1;
-        a1[j] += g0 + g1;
-        a2[j] += (g0 * v[k][0][j] + g1 * v[k][1][j]) * rstd[j];
+        if (VEC || j < nv) {                              // (tile rows past the image hold nothing)
+          float d0, d1;
+          grad_pair(k, j, d0, d1);
+          const float g0 = d0 * w0, g1 = d1 * w1;
+          a1[j] += g0 + g1;
+          a2[j] += (g0 * v[k][0][j] + g1 * v[k][1][j]) * rstd[j];
+        }
       }
     }
   }
@@ -896,19 +927,21 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
     float dw0 = 0.f, dw1 = 0.f, db0 = 0.f, db1 = 0.f;
     if (on) {
       const float w0 = wgt[2 * cp], w1 = wgt[2 * cp + 1];
-      float o0[4], o1[4];
+      float o0[4] = {0.f, 0.f, 0.f, 0.f}, o1[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float d0, d1;
-        grad_pair(k, j, d0, d1);
-        const float xh0 = v[k][0][j] * rstd[j], xh1 = v[k][1][j] * rstd[j];
-        o0[j] = rstd[j] * (d0 * w0 - m1[j] - xh0 * m2[j]);
-        o1[j] = rstd[j] * (d1 * w1 - m1[j] - xh1 * m2[j]);
-        dw0 += d0 * xh0; dw1 += d1 * xh1;
-        db0 += d0; db1 += d1;
+        if (VEC || j < nv) {
+          float d0, d1;
+          grad_pair(k, j, d0, d1);
+          const float xh0 = v[k][0][j] * rstd[j], xh1 = v[k][1][j] * rstd[j];
+          o0[j] = rstd[j] * (d0 * w0 - m1[j] - xh0 * m2[j]);
+          o1[j] = rstd[j] * (d1 * w1 - m1[j] - xh1 * m2[j]);
+          dw0 += d0 * xh0; dw1 += d1 * xh1;
+          db0 += d0; db1 += d1;
+        }
       }
-      store_quad<T>(dx + base + static_cast<size_t>(2 * cp) * t.HW, o0);
-      store_quad<T>(dx + base + static_cast<size_t>(2 * cp + 1) * t.HW, o1);
+      store_row4<T, VEC>(dx + base + static_cast<size_t>(2 * cp) * t.HW, o0, nv);
+      store_row4<T, VEC>(dx + base + static_cast<size_t>(2 * cp + 1) * t.HW, o1, nv);
     }
     dw0 = group_sum(dw0, t.gshift, lane4); dw1 = group_sum(dw1, t.gshift, lane4);
     db0 = group_sum(db0, t.gshift, lane4); db1 = group_sum(db1, t.gshift, lane4);
@@ -922,7 +955,7 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
 // Backward of the block residual on the same plan.  Grid (tiles, B); arguments as block_residual_bwd_kernel.  The NHWC
 // run of y goes through the LDS tile; each thread replaces the words it reads there by gamma * dout, and the tile leaves
 // as the contiguous run of dy.
-template <typename T, int NP>
+template <typename T, int NP, bool VEC>
 __global__ void __launch_bounds__(kBlockThreads)
 block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ y, const void* __restrict__ gamma,
                               int pdtype, T* __restrict__ dy, float* __restrict__ partial, const NormTile t,
@@ -936,7 +969,8 @@ block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ 
   const int C = t.C, C2 = C >> 1;
   const int p0 = blockIdx.x * tp, b = blockIdx.y;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
-  const bool live = 4 * g < np;
+  const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
+  const bool live = nv > 0;
   constexpr int PW = PairWord<T>::kDwords;
   const size_t base = static_cast<size_t>(b) * C * t.HW + p0 + 4 * g;
   Quad<T> q[NP][2];
@@ -944,8 +978,8 @@ block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ 
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
     if (live && cp < C2) {
-      q[k][0].load(dout + base + static_cast<size_t>(2 * cp) * t.HW);
-      q[k][1].load(dout + base + static_cast<size_t>(2 * cp + 1) * t.HW);
+      load_row4<T, VEC>(q[k][0], dout + base + static_cast<size_t>(2 * cp) * t.HW, nv);
+      load_row4<T, VEC>(q[k][1], dout + base + static_cast<size_t>(2 * cp + 1) * t.HW, nv);
     }
   }
   const int cd = C2 * PW;
@@ -965,12 +999,14 @@ block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ 
       q[k][1].get(d1);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int idx = (4 * g + j) * t.pd + cp * PW;
-        float ya, yb;
-        PairWordGet<T>::get(ldsf, idx, ya, yb);
-        dg0 += d0[j] * ya;
-        dg1 += d1[j] * yb;
-        PairWord<T>::put(ldsf, idx, g0 * d0[j], g1 * d1[j]);
+        if (VEC || j < nv) {
+          const int idx = (4 * g + j) * t.pd + cp * PW;
+          float ya, yb;
+          PairWordGet<T>::get(ldsf, idx, ya, yb);
+          dg0 += d0[j] * ya;
+          dg1 += d1[j] * yb;
+          PairWord<T>::put(ldsf, idx, g0 * d0[j], g1 * d1[j]);
+        }
       }
     }
     dg0 = group_sum(dg0, t.gshift, lane4);
