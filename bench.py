@@ -373,6 +373,32 @@ def bench_model(torch, dev, steps, warmup, batch=256):
     return res
 
 
+def bench_model_train(torch, dev, steps, warmup, batch=64):
+    """A training step (forward + backward of a scalar loss, no optimizer) of the same model in bf16, train mode, with the
+    block passes of the HIP library on both sides, and with the harness's plain torch passes for comparison."""
+    import wtconvnext.wtconvnext as M
+    res = {"workload": f"WTConvNeXt-T bf16 forward + backward, batch {batch}, 3x224x224 (no optimizer step)"}
+    x = torch.randn(batch, 3, 224, 224, device=dev).bfloat16()
+    saved = M._block_ops
+    try:
+        for tag, ops in (("hip_block_passes", saved), ("plain_torch_passes", lambda: None)):
+            M._block_ops = ops
+            torch.manual_seed(0)
+            model = M.wtconvnext_tiny().to(dev).bfloat16().train()
+
+            def step(i):
+                model(x).float().square().mean().backward()
+                for p in model.parameters():
+                    p.grad = None
+
+            wall_ms, _, _, _ = time_steps(torch, step, 1, steps, warmup)
+            res[tag] = {"ms_per_step": wall_ms, "images_per_s": batch / (wall_ms * 1e-3)}
+            del model
+    finally:
+        M._block_ops = saved
+    return res
+
+
 def model_graph_ms(torch, model, x, steps, warmup):
     """The same forward captured in one HIP graph.  Library calls inside the model (convolutions, GEMMs, the
     mean) are captured as they come, so every replay is checked against the eager logits, with eager work and a
@@ -562,6 +588,7 @@ def main():
             line["stage_sweep_bf16"] = sweep
             line["wtconv1d"] = bench_1d(torch, dev, xsteps, xwarm)
             line["wtconvnext_t"] = bench_model(torch, dev, 5, 2)
+            line["wtconvnext_t_train"] = bench_model_train(torch, dev, 5, 2)
     # the stated goal for this path: 60 % of the HBM roof for the whole step (5 * P * s bytes)
     line["target"] = {"step_frac_hbm": 0.60, "attained_fraction_of_target": main_res["step_frac_hbm"] / 0.60,
                       "note": "no published reference number exists for this metric; vs_baseline stays null"}

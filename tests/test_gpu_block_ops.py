@@ -156,6 +156,33 @@ def test_block_residual_backward(hip_device, shape, dtype, pdtype):
     check(gd.grad.float().cpu(), gr.grad.float(), f"dgamma {shape}")
 
 
+@pytest.mark.parametrize("shape", [(64, 96, 56, 56), (40, 192, 28, 28), (48, 768, 7, 7)])
+def test_block_backward_many_records_reproducible(hip_device, shape):
+    """Batches whose per-workgroup records fill every slice of the two-stage column sum (1 600 / 280 / 192 records):
+    the parameter gradients against float64 sums computed on the GPU, and bit-identical on a second run (the slices are
+    added in a fixed order; the ticket only decides which workgroup does the adding)."""
+    from wtconv_amd import block_ops
+    B, C, H, W = shape
+    gen = torch.Generator().manual_seed(C)
+    x = (torch.randn(shape, generator=gen) * 2 + 0.5).bfloat16().to(hip_device)
+    dy = torch.randn(B, H, W, C, generator=gen).bfloat16().to(hip_device)
+    w = (torch.randn(C, generator=gen) * 0.5 + 1).to(hip_device)
+    runs = [block_ops.channel_norm_backward(x, dy, w, 1e-6, True) for _ in range(2)]
+    xd = x.double()
+    xh = (xd - xd.mean(1, keepdim=True)) / torch.sqrt(xd.var(1, unbiased=False, keepdim=True) + 1e-6)
+    dyn = dy.double().permute(0, 3, 1, 2)
+    U.assert_bf16(runs[0][1].cpu(), (dyn * xh).sum((0, 2, 3)).float().cpu(), f"dweight {shape}")
+    U.assert_bf16(runs[0][2].cpu(), dyn.sum((0, 2, 3)).float().cpu(), f"dbias {shape}")
+    for a, b in zip(runs[0], runs[1]):
+        assert torch.equal(a, b)
+    gamma = (torch.randn(C, generator=gen) * 0.7).to(hip_device)
+    y = torch.randn(B, H, W, C, generator=gen).bfloat16().to(hip_device)
+    res = [block_ops.block_residual_backward(x, y, gamma) for _ in range(2)]
+    U.assert_bf16(res[0][1].cpu(), (xd * y.double().permute(0, 3, 1, 2)).sum((0, 2, 3)).float().cpu(), f"dgamma {shape}")
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(a, b)
+
+
 def test_model_training_fused_blocks_match_plain_blocks(hip_device, monkeypatch):
     """One training step of a small WTConvNeXt (fp32): loss and every parameter gradient with the fused block passes
     (forward and backward kernels) against the same model on the plain torch passes."""
