@@ -68,6 +68,8 @@ def parse():
                     help="run only the WTConv1d(64,64,5,wt_levels=4) x[64,64,4096] workload and print its line")
     ap.add_argument("--only-model", action="store_true",
                     help="run only the WTConvNeXt-T bf16 inference forward (batch 256) and print its line")
+    ap.add_argument("--only-model-train", action="store_true",
+                    help="only the training-step leg of the model (with and without the library's block passes)")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain device copy of one activation tensor (calibrates rocprof's "
                          "FETCH_SIZE/WRITE_SIZE against a kernel of known traffic) and exit")
@@ -537,6 +539,10 @@ def main():
 
     if args.only_model:
         print(json.dumps(bench_model(torch, dev, args.steps, args.warmup)))
+        return
+
+    if args.only_model_train:
+        print(json.dumps(bench_model_train(torch, dev, args.steps, args.warmup)))
         return
 
     main_res = bench_layer(torch, dev, args.dtype, args.workload, args.steps, args.warmup, per_kernel=True)
