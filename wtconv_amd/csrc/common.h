@@ -301,6 +301,14 @@ __device__ __forceinline__ void pin_values(float (&v)[N]) {
 #endif
 }
 
+// Workgroups of a launch are dealt to the eight XCDs of the GPU in turn (workgroup i runs on XCD i % 8, each with an
+// L2 of its own).  Index i of n -> an index such that the workgroups of one XCD hold a contiguous range, neighbours in
+// it being dispatched next to each other: planes that share cache lines (small planes of adjacent channels) then meet
+// in one L2.  A bijection on [0, n); the identity when n is no multiple of 8.
+__device__ __forceinline__ int xcd_contiguous(int i, int n) {
+  return (n & 7) == 0 ? (i & 7) * (n >> 3) + (i >> 3) : i;
+}
+
 // Product of two indices that fit 24 bits (rows, strides and offsets inside a plane or the
 // LDS): v_mul_i32_i24 runs at full rate, the 32-bit v_mul_lo_u32 at a quarter of it.
 __device__ __forceinline__ int imul(int a, int b) {

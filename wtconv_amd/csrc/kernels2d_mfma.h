@@ -523,8 +523,9 @@ wt2d_mfma_kernel(const T* __restrict__ x, T* __restrict__ out, const ParamTable 
   const int toff = pl.toff, upc = pl.upc, pb = pl.pb, C = pl.C, B = pl.B;
 
   const int G = gridDim.x;
-  const int u_begin = static_cast<int>(static_cast<long long>(blockIdx.x) * pl.nunits / G);
-  const int u_end = static_cast<int>(static_cast<long long>(blockIdx.x + 1) * pl.nunits / G);
+  const int wg = xcd_contiguous(blockIdx.x, G);
+  const int u_begin = static_cast<int>(static_cast<long long>(wg) * pl.nunits / G);
+  const int u_end = static_cast<int>(static_cast<long long>(wg + 1) * pl.nunits / G);
 
   PixRow<T> pf[NBL][4];
   const size_t total_elems = static_cast<size_t>(B) * C * HW;

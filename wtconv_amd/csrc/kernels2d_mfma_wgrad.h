@@ -199,7 +199,7 @@ wt2d_mfma_wgrad_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
   const int sb = wave & 3, half = wave >> 2;
   const int n = lane & 15, q = lane >> 4;
   const int H = pl.H, W = pl.W, HW = H * W, C = pl.C, B = pl.B, pb = pl.pb;
-  const int c = blockIdx.x;
+  const int c = xcd_contiguous(blockIdx.x, gridDim.x);
   const int b_begin = blockIdx.y * bchunk;
   const int b_end = b_begin + bchunk < B ? b_begin + bchunk : B;
 
