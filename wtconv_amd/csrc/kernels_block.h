@@ -37,6 +37,16 @@ __device__ __forceinline__ int div_c(int v, unsigned magic) {
 #endif
 }
 
+// The (tile, image) of a workgroup of a (tiles, B) grid, dealt so that the workgroups of one XCD hold consecutive tiles
+// (xcd_contiguous): where a tile's rows are shorter than a cache line, neighbouring tiles share lines, which then meet
+// in one L2.
+__device__ __forceinline__ void tile_of_workgroup(int& tile, int& b) {
+  const int tiles = static_cast<int>(gridDim.x);
+  const int i = xcd_contiguous(static_cast<int>(blockIdx.x) + tiles * static_cast<int>(blockIdx.y), tiles * static_cast<int>(gridDim.y));
+  b = i / tiles;
+  tile = i - b * tiles;
+}
+
 template <typename T>
 __device__ __forceinline__ void store_pair(T* p, float a, float b);
 template <> __device__ __forceinline__ void store_pair<float>(float* p, float a, float b) {
@@ -154,7 +164,9 @@ channel_norm_kernel(const T* __restrict__ x, T* __restrict__ out, const void* __
   WT_SHARED_FLOATS(ldsf);
   LT* lds = reinterpret_cast<LT*>(ldsf);         // the tile
   const int tid = threadIdx.x;
-  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * t.tp;
   const int pitch = t.tp + 1, C = t.C;
   const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
   float* psum = ldsf + t.aux;                    // [parts][tp] partial sums
@@ -279,7 +291,9 @@ channel_norm_reg_kernel(const T* __restrict__ x, T* __restrict__ out, const void
   const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
   const int g = tid & (G - 1), e = tid >> t.gshift;
   const int C = t.C, C2 = C >> 1;
-  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * tp;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
   const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
   const bool live = nv > 0;
@@ -412,7 +426,9 @@ block_residual_kernel(const T* __restrict__ y, const T* __restrict__ shortcut, c
   WT_SHARED_FLOATS(ldsf);
   T* lds = reinterpret_cast<T*>(ldsf);
   const int tid = threadIdx.x;
-  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * t.tp;
   const int pitch = t.tp + 1, C = t.C;
   const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
   const T* src = y + (static_cast<size_t>(b) * t.HW + p0) * C;
@@ -491,7 +507,9 @@ block_residual_reg_kernel(const T* __restrict__ y, const T* __restrict__ shortcu
   const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
   const int g = tid & (G - 1), e = tid >> t.gshift;
   const int C = t.C, C2 = C >> 1;
-  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * tp;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
   const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
   const bool live = nv > 0;
@@ -609,7 +627,9 @@ channel_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy, const
                         float eps, int dy_nhwc, T* __restrict__ dx, float* __restrict__ partial, const BlockTile t) {
   WT_SHARED_FLOATS(ldsf);
   const int tid = threadIdx.x;
-  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * t.tp;
   const int pitch = t.tp + 1, C = t.C;
   const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
   T* xt = reinterpret_cast<T*>(ldsf);            // tile of x, later of dx
@@ -663,7 +683,7 @@ channel_norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ dy, const
   for (int k = 0; k < parts; ++k) { m1 += psum[k * t.tp + p]; m2 += pvar[k * t.tp + p]; }
   m1 *= invC; m2 *= invC;
   // per-channel sums over the tile's pixels (before x's tile is overwritten with dx)
-  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * 2 * C;
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + tile) * 2 * C;
   for (int c = tid; c < C; c += kBlockThreads) {
     float dw = 0.f, db = 0.f;
     for (int pp = 0; pp < np; ++pp) {
@@ -695,7 +715,9 @@ block_residual_bwd_kernel(const T* __restrict__ dout, const T* __restrict__ y, c
                           T* __restrict__ dy, float* __restrict__ partial, const BlockTile t) {
   WT_SHARED_FLOATS(ldsf);
   const int tid = threadIdx.x;
-  const int p0 = blockIdx.x * t.tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * t.tp;
   const int pitch = t.tp + 1, C = t.C;
   const int np = t.HW - p0 < t.tp ? t.HW - p0 : t.tp;
   T* dt = reinterpret_cast<T*>(ldsf);            // tile of dout
@@ -706,7 +728,7 @@ block_residual_bwd_kernel(const T* __restrict__ dout, const T* __restrict__ y, c
   tile_from_nhwc<T>(y + run, yt, t, np, tid);
   for (int c = tid; c < C; c += kBlockThreads) wgt[c] = load_param(gamma, pdtype, c);
   __syncthreads();
-  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * C;
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + tile) * C;
   for (int c = tid; c < C; c += kBlockThreads) {
     float dg = 0.f;
     for (int pp = 0; pp < np; ++pp) dg = fmaf(to_f32<T>(dt[c * pitch + pp]), to_f32<T>(yt[c * pitch + pp]), dg);
@@ -802,7 +824,9 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
   const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
   const int g = tid & (G - 1), e = tid >> t.gshift;
   const int C = t.C, C2 = C >> 1;
-  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * tp;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
   const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
   const bool live = nv > 0;
@@ -919,7 +943,7 @@ channel_norm_bwd_reg_kernel(const T* __restrict__ x, const T* __restrict__ dy, c
     m1[j] = total(part + 8 * tp, j) * inv_c;
     m2[j] = total(part + 12 * tp, j) * inv_c;
   }
-  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * 2 * C;
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + tile) * 2 * C;
 #pragma unroll
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
@@ -967,7 +991,9 @@ block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ 
   const int G = 1 << t.gshift, tp = 4 * G, cs = kBlockThreads >> t.gshift;
   const int g = tid & (G - 1), e = tid >> t.gshift;
   const int C = t.C, C2 = C >> 1;
-  const int p0 = blockIdx.x * tp, b = blockIdx.y;
+  int tile, b;
+  tile_of_workgroup(tile, b);
+  const int p0 = tile * tp;
   const int np = t.HW - p0 < tp ? t.HW - p0 : tp;
   const int nv = np - 4 * g < 0 ? 0 : (np - 4 * g > 4 ? 4 : np - 4 * g);      // this thread's pixels inside the tile
   const bool live = nv > 0;
@@ -987,7 +1013,7 @@ block_residual_bwd_reg_kernel(const T* __restrict__ dout, const T* __restrict__ 
   tile_from_run(reinterpret_cast<const uint32_t*>(y + run), reinterpret_cast<uint32_t*>(ldsf), np * cd, cd, t, tid);
   __syncthreads();
   const int lane4 = lane << 2;
-  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + blockIdx.x) * C;
+  float* rec = partial + (static_cast<size_t>(b) * gridDim.x + tile) * C;
 #pragma unroll
   for (int k = 0; k < NP; ++k) {
     const int cp = e + k * cs;
