@@ -301,6 +301,30 @@ __device__ __forceinline__ void pin_values(float (&v)[N]) {
 #endif
 }
 
+// 16-byte global accesses of data that is touched once (activations streaming through a kernel): marked
+// non-temporal, so that they do not displace what the caches should keep.
+__device__ __forceinline__ uint4 load_stream_u4(const void* p) {
+#ifdef WT_EMULATE
+  return *reinterpret_cast<const uint4*>(p);
+#else
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  uint4 r;
+  r.x = v.x; r.y = v.y; r.z = v.z; r.w = v.w;
+  return r;
+#endif
+}
+__device__ __forceinline__ void store_stream_u4(void* p, const uint4& q) {
+#ifdef WT_EMULATE
+  *reinterpret_cast<uint4*>(p) = q;
+#else
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  u32x4_t v;
+  v.x = q.x; v.y = q.y; v.z = q.z; v.w = q.w;
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(p));
+#endif
+}
+
 // Workgroups of a launch are dealt to the eight XCDs of the GPU in turn (workgroup i runs on XCD i % 8, each with an
 // L2 of its own).  Index i of n -> an index such that the workgroups of one XCD hold a contiguous range, neighbours in
 // it being dispatched next to each other: planes that share cache lines (small planes of adjacent channels) then meet

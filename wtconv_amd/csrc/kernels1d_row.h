@@ -87,7 +87,9 @@ struct Row1D {
 // the workgroup has at least as many threads as lanes that hold samples), row1d_commit
 // converts and writes them to the slots.  Fast path only: rows are 16-byte sized and aligned,
 // so every vector lies wholly inside or wholly outside the row.
-template <typename T, int S>
+// STREAM: the loads are marked non-temporal (measured: pays in the whole-backward kernel, which reads two rows per
+// row it writes, not in the forward kernel).
+template <typename T, int S, bool STREAM = false>
 __device__ __forceinline__ void row1d_fetch(const T* __restrict__ row, int N, int tid, int nth,
                                             uint4 (&q)[S / (16 / sizeof(T))]) {
   constexpr int EV = 16 / sizeof(T);
@@ -95,7 +97,10 @@ __device__ __forceinline__ void row1d_fetch(const T* __restrict__ row, int N, in
   for (int u = 0; u < S / EV; ++u) {
     const int p = (tid + u * nth) * EV;
     q[u].x = 0u; q[u].y = 0u; q[u].z = 0u; q[u].w = 0u;
-    if (p < N) q[u] = *reinterpret_cast<const uint4*>(row + p);
+    if (p < N) {
+      if constexpr (STREAM) q[u] = load_stream_u4(row + p);
+      else q[u] = *reinterpret_cast<const uint4*>(row + p);
+    }
   }
 }
 
@@ -226,7 +231,7 @@ __device__ __forceinline__ void row1d_unstage(T* __restrict__ row, const float* 
           qq[k] = pack2<T>(vals[2 * k], vals[2 * k + 1]);
         q.x = qq[0]; q.y = qq[1]; q.z = qq[2]; q.w = qq[3];
       }
-      *reinterpret_cast<uint4*>(row + p) = q;
+      store_stream_u4(row + p, q);       // written once, read by another kernel: non-temporal
     } else {
 #pragma unroll
       for (int k = 0; k < EV; ++k)
@@ -861,8 +866,8 @@ __global__ __launch_bounds__(kRow1dBwdMaxLanes, 2) void wt1d_row_bwd_kernel(cons
   if (b_first < b_end && ahead) {
     const size_t r0 = (static_cast<size_t>(b_first) * pl.C + c) * pl.N;
     if constexpr (kAhead) {
-      row1d_fetch<T, S>(x + r0, pl.N, tid, nth, qx);
-      row1d_fetch<T, S>(g + r0, pl.N, tid, nth, qg);
+      row1d_fetch<T, S, true>(x + r0, pl.N, tid, nth, qx);
+      row1d_fetch<T, S, true>(g + r0, pl.N, tid, nth, qg);
       row1d_commit<T, S, SLOT>(xlds, pl.nl, tid, nth, qx);
       row1d_commit<T, S, SLOT>(glds, pl.nl, tid, nth, qg);
     }
@@ -891,8 +896,8 @@ __global__ __launch_bounds__(kRow1dBwdMaxLanes, 2) void wt1d_row_bwd_kernel(cons
     }
     if constexpr (kAhead) {
       if (ahead && more) {
-        row1d_fetch<T, S>(x + rnext, pl.N, tid, nth, qx);
-        row1d_fetch<T, S>(g + rnext, pl.N, tid, nth, qg);
+        row1d_fetch<T, S, true>(x + rnext, pl.N, tid, nth, qx);
+        row1d_fetch<T, S, true>(g + rnext, pl.N, tid, nth, qg);
       }
     }
     row1d_publish<K, S, 0>(xslot, xs);
