@@ -156,8 +156,8 @@ class WTConvNode : public torch::autograd::Function<WTConvNode> {
     const int dt = dtype_code(x.scalar_type()), pdt = dtype_code(base_w.scalar_type());
     Tensor grad_x;
     if (need_x) grad_x = at::empty_like(x, at::MemoryFormat::Contiguous);
-    // parameter gradients are written as fp32: in place for fp32 parameters, else into one flat buffer that is
-    // cast once
+    // parameter gradients are written as fp32 into one flat buffer (one allocation for the 5 + 2 L tensors): fp32
+    // parameters get views of it in their own shapes, others views of one cast of it
     const bool f32 = base_w.scalar_type() == at::kFloat;
     std::vector<Tensor> views(3 + 2 * L);      // base_w, base_b, base_s, levels
     Tensor flat;
@@ -165,20 +165,16 @@ class WTConvNode : public torch::autograd::Function<WTConvNode> {
     if (need_params) {
       std::vector<const Tensor*> plist = {&base_w, &base_b, &base_s};
       for (int i = 0; i < 2 * L; ++i) plist.push_back(&wt[i]);
-      if (f32) {
-        for (size_t i = 0; i < plist.size(); ++i)
-          if (plist[i]->defined()) views[i] = at::empty_like(*plist[i], at::MemoryFormat::Contiguous);
-      } else {
-        int64_t total = 0;
-        for (const Tensor* t : plist) total += t->defined() ? t->numel() : 0;
-        flat = at::empty({total}, x.options().dtype(at::kFloat));
-        int64_t pos = 0;
-        for (size_t i = 0; i < plist.size(); ++i)
-          if (plist[i]->defined()) {
-            views[i] = flat.narrow(0, pos, plist[i]->numel());
-            pos += plist[i]->numel();
-          }
-      }
+      int64_t total = 0;
+      for (const Tensor* t : plist) total += t->defined() ? t->numel() : 0;
+      flat = at::empty({total}, x.options().dtype(at::kFloat));
+      int64_t pos = 0;
+      for (size_t i = 0; i < plist.size(); ++i)
+        if (plist[i]->defined()) {
+          views[i] = flat.narrow(0, pos, plist[i]->numel());
+          if (f32) views[i] = views[i].view(plist[i]->sizes());
+          pos += plist[i]->numel();
+        }
       const at::TensorList lv(views.data() + 3, 2 * L);
       fill(gt, views[0], views[1], views[2], lv, L);
     }
