@@ -271,6 +271,12 @@ __device__ __forceinline__ void row1d_write_slot(float* __restrict__ slot, const
   }
 }
 
+// Scaling.  The butterflies here are sums and differences without their 1/sqrt(2): level l's coefficients are
+// 2^(l/2) times the orthonormal ones of wtconv/util/wavelet.py:46-59.  The folded weights of level l carry 2^-l
+// (row1d_fold), which makes every level's reconstruction come out exactly scaled -- each inverse butterfly and each
+// repeat of a coarse value owes 2^(-1/2), l of them in all -- and the correlation sums of level l (two pyramids, each
+// 2^(l/2) up) are brought back by 2^-l when they leave the registers (row1d_store_partial).  Only powers of two are
+// moved, which is exact; the 2 n multiplications per level and pass, and their roundings, are gone.
 // The lane's pyramid: level l (1-based) has S >> l low-pass and as many high-pass entries.
 template <int S, int L>
 struct RowPyramid {
@@ -286,8 +292,8 @@ __device__ __forceinline__ void row1d_analysis(const float (&x)[S], RowPyramid<S
     for (int q = 0; q < (S >> (l + 1)); ++q) {
       const float e = l == 0 ? x[2 * q] : py.lo[l > 0 ? l - 1 : 0][2 * q];
       const float o = l == 0 ? x[2 * q + 1] : py.lo[l > 0 ? l - 1 : 0][2 * q + 1];
-      py.lo[l][q] = (e + o) * kInvSqrt2;
-      py.hi[l][q] = (e - o) * kInvSqrt2;
+      py.lo[l][q] = e + o;
+      py.hi[l][q] = e - o;
     }
   }
 }
@@ -405,7 +411,8 @@ __device__ __forceinline__ void row1d_fold(const ParamTable& p, int pdtype, int 
     for (int l = 0; l < L; ++l) {
       if (f >= 1 + 2 * l && f < 3 + 2 * l) {
         const int ch = c * 2 + (f - 1 - 2 * l);
-        v = load_param(p.wt_weight[l], pdtype, ch * K + ts) * load_param(p.wt_scale[l], pdtype, ch);
+        v = load_param(p.wt_weight[l], pdtype, ch * K + ts) * load_param(p.wt_scale[l], pdtype, ch) *
+            (1.f / static_cast<float>(2 << l));          // 2^-(level): see "Scaling"
       }
     }
     return v;
@@ -447,14 +454,14 @@ __device__ __forceinline__ void row1d_synth(const RowPyramid<S, L>& py, const fl
     if constexpr (l > 1) {
 #pragma unroll
       for (int q = 0; q < n; ++q) {
-        zc[2 * q] = (ylo[q] + yhi[q]) * kInvSqrt2;       // ylo[q] was read from zc[q] before: q <= 2q
-        zc[2 * q + 1] = (ylo[q] - yhi[q]) * kInvSqrt2;
+        zc[2 * q] = ylo[q] + yhi[q];       // ylo[q] was read from zc[q] before: q <= 2q
+        zc[2 * q + 1] = ylo[q] - yhi[q];
       }
     } else {
 #pragma unroll
       for (int q = 0; q < n; ++q) {
-        out[2 * q] += (ylo[q] + yhi[q]) * kInvSqrt2;
-        out[2 * q + 1] += (ylo[q] - yhi[q]) * kInvSqrt2;
+        out[2 * q] += ylo[q] + yhi[q];
+        out[2 * q + 1] += ylo[q] - yhi[q];
       }
     }
     row1d_synth<K, S, SLOT, L, l - 1>(py, region, tid, nth, fwc, zc, out);
@@ -481,8 +488,8 @@ __device__ __forceinline__ void row1d_wgrad_levels(const RowPyramid<S, L>& py, c
   float glo[n], ghi[n];
 #pragma unroll
   for (int q = 0; q < n; ++q) {
-    glo[q] = (gprev[2 * q] + gprev[2 * q + 1]) * kInvSqrt2;
-    ghi[q] = (gprev[2 * q] - gprev[2 * q + 1]) * kInvSqrt2;
+    glo[q] = gprev[2 * q] + gprev[2 * q + 1];
+    ghi[q] = gprev[2 * q] - gprev[2 * q + 1];
   }
   {
     float ext[n + 2 * R];
@@ -508,7 +515,8 @@ __device__ __forceinline__ void row1d_store_partial(const float (&acc)[NF][K], f
   for (int f = 0; f < NF; ++f)
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const float v = wave_sum(acc[f][k]);
+      // the sums of level l were formed from coefficients 2^(l/2) times the orthonormal ones on either side
+      const float v = wave_sum(acc[f][k]) * (f == 0 ? 1.f : 1.f / static_cast<float>(2 << ((f - 1) / 2)));
       if (lane == 0) red[wave * NRED + f * K + k] = v;
     }
   {
@@ -534,8 +542,8 @@ __device__ __forceinline__ void row1d_publish_chain(float* __restrict__ slot, co
   float lo[n], hi[n];
 #pragma unroll
   for (int q = 0; q < n; ++q) {
-    lo[q] = (prev[2 * q] + prev[2 * q + 1]) * kInvSqrt2;
-    hi[q] = (prev[2 * q] - prev[2 * q + 1]) * kInvSqrt2;
+    lo[q] = prev[2 * q] + prev[2 * q + 1];
+    hi[q] = prev[2 * q] - prev[2 * q + 1];
   }
   row1d_publish<K, S, 1 + 2 * (l - 1)>(slot, lo);
   row1d_publish<K, S, 2 + 2 * (l - 1)>(slot, hi);
@@ -564,10 +572,10 @@ __device__ __forceinline__ void row1d_bwd_levels(const float* __restrict__ xregi
     float xhi[n], ghi[n];
 #pragma unroll
     for (int q = 0; q < n; ++q) {
-      xlo[q] = (xprev[2 * q] + xprev[2 * q + 1]) * kInvSqrt2;
-      xhi[q] = (xprev[2 * q] - xprev[2 * q + 1]) * kInvSqrt2;
-      glo[q] = (gprev[2 * q] + gprev[2 * q + 1]) * kInvSqrt2;
-      ghi[q] = (gprev[2 * q] - gprev[2 * q + 1]) * kInvSqrt2;
+      xlo[q] = xprev[2 * q] + xprev[2 * q + 1];
+      xhi[q] = xprev[2 * q] - xprev[2 * q + 1];
+      glo[q] = gprev[2 * q] + gprev[2 * q + 1];
+      ghi[q] = gprev[2 * q] - gprev[2 * q + 1];
     }
     {
       float ext[n + 2 * R];
@@ -592,14 +600,11 @@ __device__ __forceinline__ void row1d_bwd_levels(const float* __restrict__ xregi
     row1d_extend<K, S, SLOT, A>(gregion, tid, nth, glo, ext);
     row1d_conv<K, L, A, n>(ext, fwc, ylo);
   }
-  // one inverse butterfly (1/sqrt2), then l - 1 repeats (1/sqrt2 each)
-  float scale = kInvSqrt2;
-#pragma unroll
-  for (int i = 1; i < l; ++i) scale *= kInvSqrt2;
+  // (one inverse butterfly and l - 1 repeats: no factor left, see "Scaling" above)
   constexpr int REP = 1 << (l - 1);
 #pragma unroll
   for (int q = 0; q < n; ++q) {
-    const float ev = (ylo[q] + yhi[q]) * scale, od = (ylo[q] - yhi[q]) * scale;
+    const float ev = ylo[q] + yhi[q], od = ylo[q] - yhi[q];
 #pragma unroll
     for (int r = 0; r < REP; ++r) {
       o[(2 * q) * REP + r] += ev;
@@ -626,8 +631,8 @@ __device__ __forceinline__ void row1d_fwd_levels(const RowEdges<K, L>& ed, const
     float xhi[n];
 #pragma unroll
     for (int q = 0; q < n; ++q) {
-      xlo[q] = (xprev[2 * q] + xprev[2 * q + 1]) * kInvSqrt2;
-      xhi[q] = (xprev[2 * q] - xprev[2 * q + 1]) * kInvSqrt2;
+      xlo[q] = xprev[2 * q] + xprev[2 * q + 1];
+      xhi[q] = xprev[2 * q] - xprev[2 * q + 1];
     }
     float ext[n + 2 * R];
     row1d_extend_with<K, S, L, A + 1>(ed, xhi, ext);
@@ -638,13 +643,10 @@ __device__ __forceinline__ void row1d_fwd_levels(const RowEdges<K, L>& ed, const
     row1d_extend_with<K, S, L, A>(ed, xlo, ext);
     row1d_conv<K, L, A, n>(ext, fwc, ylo);
   }
-  float scale = kInvSqrt2;
-#pragma unroll
-  for (int i = 1; i < l; ++i) scale *= kInvSqrt2;
   constexpr int REP = 1 << (l - 1);
 #pragma unroll
   for (int q = 0; q < n; ++q) {
-    const float ev = (ylo[q] + yhi[q]) * scale, od = (ylo[q] - yhi[q]) * scale;
+    const float ev = ylo[q] + yhi[q], od = ylo[q] - yhi[q];
 #pragma unroll
     for (int r = 0; r < REP; ++r) {
       o[(2 * q) * REP + r] += ev;
